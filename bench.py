@@ -1,0 +1,171 @@
+#!/usr/bin/env python3
+"""Benchmark of the BERT forward pass on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C1] [--no-cpu]
+
+A step is one forward pass of the workload (default C1: BERT-base fp32, batch 128, seq_len 32,
+the configuration the headline metric is quoted on) on inputs already resident in device memory.
+Prints ONE JSON line: sequences/s over the K timed steps, the roofline of the dominant fused
+kernel (bias+GELU) measured with HIP events around its launches inside the timed steps, and the
+CPU oracle timed on this host's cores on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def algorithmic_bytes(cfg):
+    """Minimum HBM traffic per launch of each fused kernel (bytes): every operand once."""
+    m = cfg["model"]
+    B, S = cfg["batch"], cfg["seq_length"]
+    H, I, A = m["hidden"], m["intermediate"], m["heads"]
+    e = 4 if cfg["dtype"] == "f32" else 2
+    M = B * S
+    return {
+        "embed_ln": 2 * M * H * e + 5 * M + (S + 4) * H * e,
+        "bias_res_ln": 3 * M * H * e + 3 * H * e,
+        "bias_gelu": 2 * M * I * e + I * e,
+        "mask_scale_softmax": 2 * B * A * S * S * e + B * S,
+        "bias_tanh": 2 * B * H * e + H * e,
+        "mean_pool": (M + B) * H * e,
+        "row_softmax": 2 * B * cfg["labels"] * e,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="C1")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--all-kernels", action="store_true", help="time every kernel kind in an extra untimed pass")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (replicas on several GPUs share nothing); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import cubert_amd
+    from cubert_amd.testing import CONFIGS, config_inputs, config_weights
+
+    cfg = CONFIGS[args.workload]
+    m = cfg["model"]
+    B, S = cfg["batch"], cfg["seq_length"]
+    half = cfg["dtype"] == "f16"
+    w = config_weights(args.workload, seed=0)
+    ids, mask, seg = config_inputs(args.workload, seed=0)
+
+    bert = cubert_amd.Bert(w, B, S, m["layers"], m["heads"], 1 if half else 0)
+    bert.compute(ids, mask, seg)  # uploads the inputs; they stay resident
+    bert.synchronize()
+    for _ in range(args.warmup):
+        bert.compute_resident(B)
+    bert.synchronize()
+
+    # ---- timed region: K device-resident forward passes; the dominant fused kernel is bracketed by events
+    dominant = "bias_gelu"
+    bert.profile([dominant])
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        bert.compute_resident(B)
+    bert.synchronize()
+    t1 = time.perf_counter()
+    prof = bert.profile_read()
+    bert.profile([])
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = B / (ms_per_step * 1e-3)
+
+    alg = algorithmic_bytes(cfg)
+    total_ms, launches = prof[dominant]
+    avg_us = total_ms * 1e3 / launches
+    achieved = alg[dominant] / (avg_us * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "algorithmic_bytes_per_launch": alg[dominant], "avg_launch_us": round(avg_us, 2), "launches": launches}
+
+    # ---- every kernel kind, in an extra untimed pass (reported, not part of `value`)
+    kernels = {}
+    if args.all_kernels:
+        bert.profile([k for k in bert.KINDS])
+        for _ in range(max(5, args.steps // 5)):
+            bert.compute_resident(B)
+        for k, (ms, n) in bert.profile_read().items():
+            us = ms * 1e3 / n
+            kernels[k] = {"avg_us": round(us, 2), "launches": n}
+            if k in alg:
+                kernels[k]["GB/s"] = round(alg[k] / (us * 1e-6) / 1e9, 1)
+                kernels[k]["frac_hbm_peak"] = round(alg[k] / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
+        bert.profile([])
+
+    # ---- the public path: host arrays in, host array out (PCIe-inclusive), and p50 latency at batch 1
+    out = np.empty((B, m["hidden"]), np.float16 if half else np.float32)
+    o = cubert_amd.Output(out, cubert_amd.OutputType.POOLED_OUTPUT)
+    lat = []
+    for i in range(10 + 30):
+        t = time.perf_counter()
+        bert.compute(ids, mask, seg)
+        bert.output(B, o)
+        if i >= 10:
+            lat.append((time.perf_counter() - t) * 1e3)
+    host_path = {"mean_ms": round(float(np.mean(lat)), 3), "p50_ms": round(float(np.median(lat)), 3),
+                 "sequences_per_s": round(B / (np.mean(lat) * 1e-3), 1), "output": "POOLED_OUTPUT"}
+    lat1 = []
+    for i in range(20 + 100):
+        t = time.perf_counter()
+        bert.compute(ids[:1], mask[:1], seg[:1])
+        bert.output(1, o)
+        if i >= 20:
+            lat1.append((time.perf_counter() - t) * 1e3)
+    p50_b1 = round(float(np.median(lat1)), 3)
+    bert.close()
+
+    # ---- CPU baseline: the oracle (a port of the reference's CPU path) on this host's cores
+    cpu = None
+    if not args.no_cpu:
+        import oracle
+        threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        oracle.lib()
+        oracle.set_blas_threads(threads)
+        wf = {k: oracle.round_to_half(v) for k, v in w.items()} if half else w
+        vars_obj = oracle.Vars(wf)
+        # bounded sample: at most 128 sequences of the workload per pass, 1 warm-up + up to 3 timed passes or ~20 s
+        n = min(B, 128)
+        oracle.bert_forward(wf, ids[:n], mask[:n], seg[:n], m["layers"], m["heads"], vars_obj=vars_obj)
+        times = []
+        start = time.perf_counter()
+        while len(times) < 3 and time.perf_counter() - start < 20:
+            t = time.perf_counter()
+            oracle.bert_forward(wf, ids[:n], mask[:n], seg[:n], m["layers"], m["heads"], vars_obj=vars_obj)
+            times.append(time.perf_counter() - t)
+        cpu = {"value": round(n / float(np.mean(times)), 2), "unit": "sequences/s", "cores": threads, "kind": "port",
+               "sample": "%d pass(es) of %d sequences of %s (seq_len %d), fp32, mean %.1f ms/pass" %
+                         (len(times), n, args.workload, S, float(np.mean(times)) * 1e3),
+               "blas": os.path.basename(oracle.blas_name())}
+
+    line = {
+        "metric": "sequences/s, BERT forward pass (%s)" % args.workload,
+        "value": round(value, 1), "unit": "sequences/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": cfg["dtype"], "data": "synthetic",
+        "config": {"workload": "%s: %s %s batch %d seq_len %d, random-init N(0,0.02) weights, inputs resident in HBM" %
+                               (args.workload, "BERT-large" if m["hidden"] == 1024 else "BERT-base", cfg["dtype"], B, S)},
+        "roofline": roofline, "cpu_baseline": cpu,
+        "p50_ms_batch1_host_path": p50_b1, "host_path": host_path,
+    }
+    if kernels:
+        line["kernels"] = kernels
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,238 @@
+#include "Bert.h"
+
+#include <iostream>
+#include <stdexcept>
+#include <vector>
+
+namespace cuBERT {
+
+template <typename T>
+Bert<T>::Bert(const std::unordered_map<std::string, T *> &var, size_t max_batch_size, size_t seq_length,
+              size_t vocab_size, size_t type_vocab_size, size_t hidden_size, size_t num_hidden_layers,
+              size_t num_attention_heads, size_t intermediate_size, size_t num_labels)
+        : max_batch_size(max_batch_size), seq_length(seq_length), hidden_size(hidden_size), num_labels(num_labels),
+          transformer(nullptr), _sequence_output(nullptr) {
+    this->stream = cuBERT::cuda_stream_create();
+    this->cublas = cuBERT::blas_create();
+    cuBERT::blas_set_stream(cublas, stream);
+
+    has_pooler_dense = var.count("bert/pooler/dense/kernel") != 0;
+    has_classifier = var.count("output_weights") != 0;
+    has_classifier_bias = has_classifier && var.count("output_bias") != 0;
+
+    const size_t H = hidden_size;
+    layout_weights(vocab_size, type_vocab_size);
+    weights.allocate();
+    layout_weights(vocab_size, type_vocab_size);
+
+    cuBERT::memcpy(word_embeddings, var.at("bert/embeddings/word_embeddings"), vocab_size * H * sizeof(T), 1);
+    cuBERT::memcpy(token_type_embeddings, var.at("bert/embeddings/token_type_embeddings"),
+                   type_vocab_size * H * sizeof(T), 1);
+    // only the positions a sequence of seq_length tokens can use are kept on the device
+    cuBERT::memcpy(position_embeddings, var.at("bert/embeddings/position_embeddings"), seq_length * H * sizeof(T), 1);
+    cuBERT::memcpy(embedding_norm_beta, var.at("bert/embeddings/LayerNorm/beta"), H * sizeof(T), 1);
+    cuBERT::memcpy(embedding_norm_gamma, var.at("bert/embeddings/LayerNorm/gamma"), H * sizeof(T), 1);
+    if (has_pooler_dense) {
+        cuBERT::memcpy(pooler_kernel, var.at("bert/pooler/dense/kernel"), H * H * sizeof(T), 1);
+        cuBERT::memcpy(pooler_bias, var.at("bert/pooler/dense/bias"), H * sizeof(T), 1);
+    }
+    if (has_classifier) {
+        cuBERT::memcpy(output_weights, var.at("output_weights"), num_labels * H * sizeof(T), 1);
+        if (has_classifier_bias) cuBERT::memcpy(output_bias, var.at("output_bias"), num_labels * sizeof(T), 1);
+    }
+
+    this->transformer = new Transformer<T>(cublas, "bert/encoder", var, max_batch_size, seq_length, hidden_size,
+                                           num_hidden_layers, num_attention_heads, intermediate_size);
+    this->transformer->set_profiler(&profiler);
+
+    layout_buffers();
+    buffers.allocate();
+    layout_buffers();
+}
+
+template <typename T>
+Bert<T>::~Bert() {
+    cuBERT::cuda_stream_synchronize(stream);
+    delete transformer;
+    cuBERT::blas_destroy(cublas);
+    cuBERT::cuda_stream_destroy(stream);
+}
+
+template <typename T>
+void Bert<T>::layout_weights(size_t vocab_size, size_t type_vocab_size) {
+    const size_t H = hidden_size;
+    word_embeddings = weights.take<T>(vocab_size * H);
+    token_type_embeddings = weights.take<T>(type_vocab_size * H);
+    position_embeddings = weights.take<T>(seq_length * H);
+    embedding_norm_beta = weights.take<T>(H);
+    embedding_norm_gamma = weights.take<T>(H);
+    pooler_kernel = has_pooler_dense ? weights.take<T>(H * H) : nullptr;
+    pooler_bias = has_pooler_dense ? weights.take<T>(H) : nullptr;
+    output_weights = has_classifier ? weights.take<T>(num_labels * H) : nullptr;
+    output_bias = has_classifier_bias ? weights.take<T>(num_labels) : nullptr;
+}
+
+template <typename T>
+void Bert<T>::layout_buffers() {
+    const size_t M = max_batch_size * seq_length;
+    input_ids_buf = buffers.take<int>(M);
+    input_mask_buf = buffers.take<int8_t>(M);
+    segment_ids_buf = buffers.take<int8_t>(M);
+    _embedding_output = buffers.take<T>(M * hidden_size);
+    _pooled_output = buffers.take<T>(max_batch_size * hidden_size);
+    _logits = has_classifier ? buffers.take<T>(max_batch_size * num_labels) : nullptr;
+    _probs = has_classifier ? buffers.take<T>(max_batch_size * num_labels) : nullptr;
+}
+
+template <typename T>
+void Bert<T>::_pre_compute(size_t) {}
+
+template <typename T>
+void Bert<T>::compute(size_t batch_size, int *input_ids, int8_t *input_mask, int8_t *segment_ids) {
+    if (batch_size > max_batch_size) {
+        throw std::invalid_argument("batch_size > max_batch_size");
+    } else if (batch_size == 0) {
+        return;
+    }
+    const size_t M = batch_size * seq_length;
+    cuBERT::memcpyAsync(input_ids_buf, input_ids, sizeof(int) * M, 1, stream);
+    cuBERT::memcpyAsync(input_mask_buf, input_mask, sizeof(int8_t) * M, 1, stream);
+    cuBERT::memcpyAsync(segment_ids_buf, segment_ids, sizeof(int8_t) * M, 1, stream);
+    forward(batch_size);
+}
+
+template <typename T>
+void Bert<T>::compute_resident(size_t batch_size) {
+    if (batch_size > max_batch_size) {
+        throw std::invalid_argument("batch_size > max_batch_size");
+    } else if (batch_size == 0) {
+        return;
+    }
+    forward(batch_size);
+}
+
+template <typename T>
+void Bert<T>::forward(size_t batch_size) {
+    const int B = (int) batch_size, S = (int) seq_length, H = (int) hidden_size, L = (int) num_labels;
+
+    // bert/embeddings
+    {
+        Timed t(&profiler, Profiler::kEmbedLayerNorm, stream);
+        cuBERT::embed_layer_norm(input_ids_buf, segment_ids_buf, word_embeddings, position_embeddings,
+                                 token_type_embeddings, embedding_norm_beta, embedding_norm_gamma, _embedding_output,
+                                 B, S, H, stream);
+    }
+
+    // bert/encoder
+    _sequence_output = transformer->_in_compute(batch_size, _embedding_output, input_mask_buf);
+
+    // bert/pooler
+    if (has_pooler_dense) {
+        // first token of every sequence: the B rows are seq_length*hidden apart
+        {
+            Timed t(&profiler, Profiler::kDenseGemm, stream);
+            cuBERT::blas_gemm(cublas, false, false, H, B, H, 1.f, pooler_kernel, H, _sequence_output, H * S, 0.f,
+                              _pooled_output, H);
+        }
+        Timed t(&profiler, Profiler::kBiasTanh, stream);
+        cuBERT::tanh_(_pooled_output, pooler_bias, B, H, stream);
+    } else {
+        Timed t(&profiler, Profiler::kMeanPool, stream);
+        cuBERT::reduce_mean_1(_sequence_output, _pooled_output, B, S, H, stream);
+    }
+
+    if (has_classifier) {
+        // logits = pooled * W^T (+ bias), W is [num_labels, hidden] row-major
+        {
+            Timed t(&profiler, Profiler::kDenseGemm, stream);
+            cuBERT::blas_gemm(cublas, true, false, L, B, H, 1.f, output_weights, H, _pooled_output, H, 0.f, _logits, L,
+                              output_bias);
+        }
+        Timed t(&profiler, Profiler::kRowSoftmax, stream);
+        cuBERT::softmax_(_logits, _probs, B, L, stream);
+    }
+}
+
+template <typename T>
+void Bert<T>::logits(size_t batch_size, T *logits, T *probs) {
+    if (!has_classifier) {
+        std::cerr << "model does not have additional_output_layer, the output logits is wrong." << std::endl;
+    }
+    if (has_classifier && logits != nullptr) {
+        cuBERT::memcpyAsync(logits, _logits, sizeof(T) * batch_size * num_labels, 2, stream);
+    }
+    if (has_classifier && probs != nullptr) {
+        cuBERT::memcpyAsync(probs, _probs, sizeof(T) * batch_size * num_labels, 2, stream);
+    }
+    cuBERT::cuda_stream_synchronize(stream);
+}
+
+template <typename T>
+void Bert<T>::pooled_output(size_t batch_size, T *pooled_output) {
+    cuBERT::memcpyAsync(pooled_output, _pooled_output, sizeof(T) * batch_size * hidden_size, 2, stream);
+    cuBERT::cuda_stream_synchronize(stream);
+}
+
+template <typename T>
+void Bert<T>::sequence_output(size_t batch_size, T *sequence_output) {
+    cuBERT::memcpyAsync(sequence_output, _sequence_output, sizeof(T) * batch_size * seq_length * hidden_size, 2, stream);
+    cuBERT::cuda_stream_synchronize(stream);
+}
+
+template <typename T>
+void Bert<T>::embedding_output(size_t batch_size, T *embedding_output) {
+    cuBERT::memcpyAsync(embedding_output, _embedding_output, sizeof(T) * batch_size * seq_length * hidden_size, 2,
+                        stream);
+    cuBERT::cuda_stream_synchronize(stream);
+}
+
+template <typename T>
+void Bert<T>::output(size_t batch_size, cuBERT_Output *output) {
+    const size_t tokens = batch_size * seq_length * hidden_size;
+    if (output->logits != nullptr && has_classifier) {
+        cuBERT::memcpyAsync(output->logits, _logits, sizeof(T) * batch_size * num_labels, 2, stream);
+    }
+    if (output->probs != nullptr && has_classifier) {
+        cuBERT::memcpyAsync(output->probs, _probs, sizeof(T) * batch_size * num_labels, 2, stream);
+    }
+    if (output->pooled_output != nullptr) {
+        cuBERT::memcpyAsync(output->pooled_output, _pooled_output, sizeof(T) * batch_size * hidden_size, 2, stream);
+    }
+    if (output->sequence_output != nullptr) {
+        cuBERT::memcpyAsync(output->sequence_output, _sequence_output, sizeof(T) * tokens, 2, stream);
+    }
+    if (output->embedding_output != nullptr) {
+        cuBERT::memcpyAsync(output->embedding_output, _embedding_output, sizeof(T) * tokens, 2, stream);
+    }
+    cuBERT::cuda_stream_synchronize(stream);
+}
+
+template <>
+void Bert<float>::output_to_float(size_t batch_size, cuBERT_Output *output) {
+    this->output(batch_size, output);
+}
+
+template <>
+void Bert<half>::output_to_float(size_t batch_size, cuBERT_Output *output) {
+    const size_t tokens = batch_size * seq_length * hidden_size;
+    std::vector<half> lg(output->logits ? batch_size * num_labels : 0), pr(output->probs ? batch_size * num_labels : 0),
+            po(output->pooled_output ? batch_size * hidden_size : 0), sq(output->sequence_output ? tokens : 0),
+            em(output->embedding_output ? tokens : 0);
+    cuBERT_Output tmp;
+    tmp.logits = output->logits ? lg.data() : nullptr;
+    tmp.probs = output->probs ? pr.data() : nullptr;
+    tmp.pooled_output = output->pooled_output ? po.data() : nullptr;
+    tmp.sequence_output = output->sequence_output ? sq.data() : nullptr;
+    tmp.embedding_output = output->embedding_output ? em.data() : nullptr;
+    this->output(batch_size, &tmp);
+    if (output->logits) half2float(lg.data(), (float *) output->logits, lg.size());
+    if (output->probs) half2float(pr.data(), (float *) output->probs, pr.size());
+    if (output->pooled_output) half2float(po.data(), (float *) output->pooled_output, po.size());
+    if (output->sequence_output) half2float(sq.data(), (float *) output->sequence_output, sq.size());
+    if (output->embedding_output) half2float(em.data(), (float *) output->embedding_output, em.size());
+}
+
+template class Bert<float>;
+template class Bert<half>;
+
+}  // namespace cuBERT

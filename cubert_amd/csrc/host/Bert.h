@@ -1,0 +1,97 @@
+// One BERT model on one device: owns a stream, a BLAS context, the device
+// copies of the weights and all activation buffers.  Public surface of the
+// reference's Bert<T> (src/cuBERT/Bert.h:17-44).  Not thread-safe; BertM
+// serialises access.
+#ifndef CUBERT_HOST_BERT_H
+#define CUBERT_HOST_BERT_H
+
+#include <cstddef>
+#include <cstdint>
+#include <string>
+#include <unordered_map>
+
+#include "Arena.h"
+#include "Transformer.h"
+#include "cuBERT.h"
+
+namespace cuBERT {
+
+template <typename T>
+class Bert {
+public:
+    // `var` maps TensorFlow variable names to host arrays (see Transformer.cpp and Bert.cpp for the
+    // names).  "bert/pooler/dense/kernel" present -> first-token dense+tanh pooler, absent -> mean
+    // pooler; "output_weights" present -> classifier head with `num_labels` rows ("output_bias" optional).
+    explicit Bert(const std::unordered_map<std::string, T *> &var, size_t max_batch_size, size_t seq_length,
+                  size_t vocab_size, size_t type_vocab_size, size_t hidden_size = 768, size_t num_hidden_layers = 12,
+                  size_t num_attention_heads = 12, size_t intermediate_size = 3072, size_t num_labels = 1);
+
+    virtual ~Bert();
+
+    Bert(const Bert &) = delete;
+    Bert &operator=(const Bert &) = delete;
+
+    // Nothing to prepare between requests in this implementation; kept so callers of the reference compile.
+    void _pre_compute(size_t batch_size);
+
+    // Copies the three host input arrays to the device and enqueues the forward pass.  Asynchronous:
+    // one of the output methods below must follow to wait for and fetch results.
+    void compute(size_t batch_size, int *input_ids, int8_t *input_mask, int8_t *segment_ids);
+
+    // Output methods: copy to host arrays (nullptr = skip) and synchronise the stream.
+    void logits(size_t batch_size, T *logits, T *probs);
+    void pooled_output(size_t batch_size, T *pooled_output);
+    void sequence_output(size_t batch_size, T *sequence_output);
+    void embedding_output(size_t batch_size, T *embedding_output);
+    void output(size_t batch_size, cuBERT_Output *output);
+    // Same, but a half model converts to float on the host first.
+    void output_to_float(size_t batch_size, cuBERT_Output *output);
+
+    // The stream all of this model's work runs on (for timing with events).
+    void *get_stream() const { return stream; }
+
+    // The forward pass again on the inputs the last compute() left on the device (no host copies):
+    // the steady-state device work of a request, used for throughput measurements.
+    void compute_resident(size_t batch_size);
+
+    // Per-kernel timing: switch kinds on (bit k = Profiler::Kind k), run, synchronise, then read.
+    void profile(unsigned kinds) { profiler.enable(kinds); }
+    void profile_read(double *total_ms, int *count) {
+        cuBERT::cuda_stream_synchronize(stream);
+        profiler.collect(total_ms, count);
+    }
+
+private:
+    void forward(size_t batch_size);
+    void layout_weights(size_t vocab_size, size_t type_vocab_size);
+    void layout_buffers();
+
+    void *cublas;
+    void *stream;
+
+    size_t max_batch_size, seq_length, hidden_size, num_labels;
+    bool has_pooler_dense, has_classifier, has_classifier_bias;
+
+    Transformer<T> *transformer;
+    Profiler profiler;
+
+    Arena weights;
+    T *word_embeddings, *token_type_embeddings, *position_embeddings;  // position: first seq_length rows only
+    T *embedding_norm_beta, *embedding_norm_gamma;
+    T *pooler_kernel, *pooler_bias;
+    T *output_weights, *output_bias;
+
+    Arena buffers;
+    int *input_ids_buf;
+    int8_t *input_mask_buf;
+    int8_t *segment_ids_buf;
+    T *_embedding_output;
+    T *_sequence_output;  // points into the transformer's buffers
+    T *_pooled_output;
+    T *_logits;
+    T *_probs;
+};
+
+}  // namespace cuBERT
+
+#endif  // CUBERT_HOST_BERT_H

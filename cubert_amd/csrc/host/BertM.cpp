@@ -1,0 +1,87 @@
+#include "BertM.h"
+
+#include <chrono>
+#include <iostream>
+#include <stdexcept>
+
+namespace cuBERT {
+
+template <typename T>
+BertM<T>::BertM(const char *model_file, size_t max_batch_size, size_t seq_length, size_t num_hidden_layers,
+                size_t num_attention_heads)
+        : seq_length(seq_length), graph(model_file), rr(0) {
+    const int count = cuBERT::get_gpu_count();
+    if (count == 0) {
+        throw std::invalid_argument("No GPU device detected");
+    }
+    std::cerr << "Found GPU count: " << count << std::endl;
+
+    for (int device = 0; device < count; ++device) {
+        const auto start = std::chrono::high_resolution_clock::now();
+        cuBERT::set_gpu(device);
+        cuBERT::gpu_info(device);
+        bert_instances.push_back(new Bert<T>(graph.var, max_batch_size, seq_length, graph.vocab_size,
+                                             graph.type_vocab_size, graph.hidden_size, num_hidden_layers,
+                                             num_attention_heads, graph.intermediate_size, graph.num_labels));
+        mutex_instances.push_back(new std::mutex());
+        const auto finish = std::chrono::high_resolution_clock::now();
+        std::cerr << "device setup: " << device << ". Took "
+                  << std::chrono::duration_cast<std::chrono::milliseconds>(finish - start).count() << " milliseconds."
+                  << std::endl;
+    }
+}
+
+template <typename T>
+BertM<T>::~BertM() {
+    for (size_t i = 0; i < bert_instances.size(); ++i) {
+        cuBERT::set_gpu((int) i);
+        delete bert_instances[i];
+    }
+    for (auto *m : mutex_instances) delete m;
+}
+
+template <typename T>
+unsigned int BertM<T>::compute(size_t batch_size, int *input_ids, int8_t *input_mask, int8_t *segment_ids, T *output,
+                               cuBERT_OutputType output_type) {
+    const uint8_t count = rr++;
+    const unsigned int choice = count % bert_instances.size();
+
+    cuBERT::set_gpu((int) choice);
+    Bert<T> *bert = bert_instances[choice];
+    std::lock_guard<std::mutex> lg(*mutex_instances[choice]);
+
+    bert->compute(batch_size, input_ids, input_mask, segment_ids);
+    switch (output_type) {
+        case cuBERT_LOGITS: bert->logits(batch_size, output, nullptr); break;
+        case cuBERT_PROBS: bert->logits(batch_size, nullptr, output); break;
+        case cuBERT_POOLED_OUTPUT: bert->pooled_output(batch_size, output); break;
+        case cuBERT_EMBEDDING_OUTPUT: bert->embedding_output(batch_size, output); break;
+        case cuBERT_SEQUENCE_OUTPUT: bert->sequence_output(batch_size, output); break;
+        default: throw std::invalid_argument("invalid output type");
+    }
+    return choice;
+}
+
+template <typename T>
+unsigned int BertM<T>::compute(size_t batch_size, int *input_ids, int8_t *input_mask, int8_t *segment_ids,
+                               cuBERT_Output *output, bool output_to_float) {
+    const uint8_t count = rr++;
+    const unsigned int choice = count % bert_instances.size();
+
+    cuBERT::set_gpu((int) choice);
+    Bert<T> *bert = bert_instances[choice];
+    std::lock_guard<std::mutex> lg(*mutex_instances[choice]);
+
+    bert->compute(batch_size, input_ids, input_mask, segment_ids);
+    if (output_to_float) {
+        bert->output_to_float(batch_size, output);
+    } else {
+        bert->output(batch_size, output);
+    }
+    return choice;
+}
+
+template class BertM<float>;
+template class BertM<half>;
+
+}  // namespace cuBERT

@@ -1,0 +1,107 @@
+// Optional per-kernel timing of a forward pass with stream events: a pair of
+// events is recorded around each launch of the kinds that are switched on, and
+// read back after the stream has been synchronised.  Off by default (no events
+// are recorded then).  The reference has no counterpart.
+#ifndef CUBERT_HOST_PROFILER_H
+#define CUBERT_HOST_PROFILER_H
+
+#include <utility>
+#include <vector>
+
+#include "common.h"
+
+namespace cuBERT {
+
+class Profiler {
+public:
+    enum Kind {
+        kEmbedLayerNorm = 0,
+        kBiasResLayerNorm = 1,
+        kBiasGelu = 2,
+        kMaskScaleSoftmax = 3,
+        kBiasTanh = 4,
+        kMeanPool = 5,
+        kRowSoftmax = 6,
+        kDenseGemm = 7,
+        kAttentionGemm = 8,
+        kKinds = 9
+    };
+
+    ~Profiler() {
+        for (auto &e : pool) {
+            cubert_event_destroy(e.first);
+            cubert_event_destroy(e.second);
+        }
+    }
+
+    // Bit k of `kinds` switches timing of Kind k on; 0 switches everything off.
+    void enable(unsigned kinds) {
+        mask = kinds;
+        if (mask != 0) grow(1024);
+    }
+
+    bool on(Kind k) const { return (mask >> k) & 1u; }
+
+    void begin(Kind k, void *stream) {
+        if (!on(k)) return;
+        if (used == pool.size()) grow(pool.size() + 1024);
+        CUBERT_CHECK(cubert_event_record(pool[used].first, stream));
+    }
+
+    void end(Kind k, void *stream) {
+        if (!on(k)) return;
+        CUBERT_CHECK(cubert_event_record(pool[used].second, stream));
+        kinds_used.push_back(k);
+        ++used;
+    }
+
+    // Adds the elapsed time of every pair recorded since the last call to total_ms[kind] / count[kind]
+    // and forgets them.  The stream must have been synchronised.
+    void collect(double *total_ms, int *count) {
+        for (size_t i = 0; i < used; ++i) {
+            float ms = 0.f;
+            CUBERT_CHECK(cubert_event_elapsed_ms(pool[i].first, pool[i].second, &ms));
+            total_ms[kinds_used[i]] += ms;
+            count[kinds_used[i]] += 1;
+        }
+        used = 0;
+        kinds_used.clear();
+    }
+
+private:
+    void grow(size_t n) {
+        while (pool.size() < n) {
+            void *a = cubert_event_create(), *b = cubert_event_create();
+            if (!a || !b) {
+                fprintf(stderr, "cuBERT: could not create timing events\n");
+                exit(EXIT_FAILURE);
+            }
+            pool.emplace_back(a, b);
+        }
+    }
+
+    unsigned mask = 0;
+    size_t used = 0;
+    std::vector<std::pair<void *, void *>> pool;
+    std::vector<Kind> kinds_used;
+};
+
+// RAII bracket around one launch; does nothing when `p` is null or the kind is off.
+class Timed {
+public:
+    Timed(Profiler *p, Profiler::Kind k, void *stream) : p(p), k(k), stream(stream) {
+        if (p) p->begin(k, stream);
+    }
+    ~Timed() {
+        if (p) p->end(k, stream);
+    }
+
+private:
+    Profiler *p;
+    Profiler::Kind k;
+    void *stream;
+};
+
+}  // namespace cuBERT
+
+#endif  // CUBERT_HOST_PROFILER_H

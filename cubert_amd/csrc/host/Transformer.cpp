@@ -1,0 +1,215 @@
+#include "Transformer.h"
+
+#include <cmath>
+#include <stdexcept>
+
+namespace cuBERT {
+
+namespace {
+template <typename T>
+void upload(T *dst, const T *src, size_t count) {
+    if (dst != nullptr) cuBERT::memcpy(dst, src, count * sizeof(T), 1);
+}
+}  // namespace
+
+template <typename T>
+Transformer<T>::Transformer(void *cublas, const std::string &var_prefix,
+                            const std::unordered_map<std::string, T *> &var, size_t max_batch_size,
+                            size_t seq_length, size_t hidden_size, size_t num_hidden_layers,
+                            size_t num_attention_heads, size_t intermediate_size)
+        : cublas(cublas), max_batch_size(max_batch_size), seq_length(seq_length), hidden_size(hidden_size),
+          num_hidden_layers(num_hidden_layers), num_attention_heads(num_attention_heads),
+          intermediate_size(intermediate_size), layers(num_hidden_layers) {
+    if (num_attention_heads == 0 || hidden_size % num_attention_heads != 0) {
+        throw std::invalid_argument("hidden_size must be a multiple of num_attention_heads");
+    }
+    const size_t H = hidden_size, I = intermediate_size;
+
+    // Weight names as the reference resolves them (Transformer.cpp:54-101, AttentionSelf.cpp:27-44);
+    // a missing name throws std::out_of_range from unordered_map::at, as it does there.
+    layout_weights();
+    weights.allocate();
+    layout_weights();
+
+    std::vector<T> packed(H * 3 * H), packed_bias(3 * H);
+    for (size_t l = 0; l < num_hidden_layers; ++l) {
+        const std::string p = var_prefix + "/layer_" + std::to_string(l);
+        const T *q = var.at(p + "/attention/self/query/kernel"), *qb = var.at(p + "/attention/self/query/bias");
+        const T *k = var.at(p + "/attention/self/key/kernel"), *kb = var.at(p + "/attention/self/key/bias");
+        const T *v = var.at(p + "/attention/self/value/kernel"), *vb = var.at(p + "/attention/self/value/bias");
+        // [in, out] row-major kernels side by side: row i = [Wq[i,:] | Wk[i,:] | Wv[i,:]]
+        for (size_t i = 0; i < H; ++i) {
+            std::memcpy(&packed[i * 3 * H], q + i * H, H * sizeof(T));
+            std::memcpy(&packed[i * 3 * H + H], k + i * H, H * sizeof(T));
+            std::memcpy(&packed[i * 3 * H + 2 * H], v + i * H, H * sizeof(T));
+        }
+        std::memcpy(&packed_bias[0], qb, H * sizeof(T));
+        std::memcpy(&packed_bias[H], kb, H * sizeof(T));
+        std::memcpy(&packed_bias[2 * H], vb, H * sizeof(T));
+        Layer &w = layers[l];
+        upload(w.qkv_kernel, packed.data(), H * 3 * H);
+        upload(w.qkv_bias, packed_bias.data(), 3 * H);
+        upload(w.attention_output_kernel, var.at(p + "/attention/output/dense/kernel"), H * H);
+        upload(w.attention_output_bias, var.at(p + "/attention/output/dense/bias"), H);
+        upload(w.attention_norm_beta, var.at(p + "/attention/output/LayerNorm/beta"), H);
+        upload(w.attention_norm_gamma, var.at(p + "/attention/output/LayerNorm/gamma"), H);
+        upload(w.intermediate_kernel, var.at(p + "/intermediate/dense/kernel"), H * I);
+        upload(w.intermediate_bias, var.at(p + "/intermediate/dense/bias"), I);
+        upload(w.output_kernel, var.at(p + "/output/dense/kernel"), I * H);
+        upload(w.output_bias, var.at(p + "/output/dense/bias"), H);
+        upload(w.output_norm_beta, var.at(p + "/output/LayerNorm/beta"), H);
+        upload(w.output_norm_gamma, var.at(p + "/output/LayerNorm/gamma"), H);
+    }
+
+    layout_buffers();
+    buffers.allocate();
+    layout_buffers();
+}
+
+template <typename T>
+void Transformer<T>::layout_weights() {
+    const size_t H = hidden_size, I = intermediate_size;
+    for (Layer &w : layers) {
+        w.qkv_kernel = weights.take<T>(H * 3 * H);
+        w.qkv_bias = weights.take<T>(3 * H);
+        w.attention_output_kernel = weights.take<T>(H * H);
+        w.attention_output_bias = weights.take<T>(H);
+        w.attention_norm_beta = weights.take<T>(H);
+        w.attention_norm_gamma = weights.take<T>(H);
+        w.intermediate_kernel = weights.take<T>(H * I);
+        w.intermediate_bias = weights.take<T>(I);
+        w.output_kernel = weights.take<T>(I * H);
+        w.output_bias = weights.take<T>(H);
+        w.output_norm_beta = weights.take<T>(H);
+        w.output_norm_gamma = weights.take<T>(H);
+    }
+}
+
+template <typename T>
+void Transformer<T>::layout_buffers() {
+    const size_t M = max_batch_size * seq_length, H = hidden_size;
+    qkv_out = buffers.take<T>(M * 3 * H);
+    attention_scores = buffers.take<T>(max_batch_size * num_attention_heads * seq_length * seq_length);
+    context_out = buffers.take<T>(M * H);
+    attention_output = buffers.take<T>(M * H);
+    intermediate_output = buffers.take<T>(M * intermediate_size);
+    layer_output[0] = buffers.take<T>(M * H);
+    layer_output[1] = buffers.take<T>(M * H);
+}
+
+template <typename T>
+T *Transformer<T>::compute(size_t batch_size, T *input_gpu, int8_t *attention_mask) {
+    _pre_compute(batch_size);
+    return _in_compute(batch_size, input_gpu, attention_mask);
+}
+
+template <typename T>
+void Transformer<T>::_pre_compute(size_t) {}
+
+// scores[b, a, q, k] = (1/sqrt d) * sum_j Q[b, q, a, j] K[b, k, a, j];  softmax with mask;
+// ctx[b, q, a, :] = sum_k p[b, a, q, k] V[b, k, a, :].   Q, K, V are column blocks of qkv[M, 3H].
+// The (b, a) problems have two strides (b: seq*3H, a: d), a strided-batched GEMM has one, so the
+// shorter of the two axes is looped on the host and the longer one is the GEMM batch.
+template <typename T>
+void Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *mask) {
+    void *stream = cuBERT::blas_get_stream(cublas);
+    const int S = (int) seq_length, A = (int) num_attention_heads, H = (int) hidden_size, d = H / A;
+    const int B = (int) batch_size, ld = 3 * H;
+    const float alpha = (float) (1.0 / std::sqrt((double) d));
+    const T *Q = qkv, *K = qkv + H, *V = qkv + 2 * H;
+    const long long seq_stride = (long long) S * ld, head_stride = d;
+    const long long score_b = (long long) A * S * S, score_a = (long long) S * S;
+
+    const bool loop_heads = A <= B;
+    const int outer = loop_heads ? A : B, inner = loop_heads ? B : A;
+    const long long in_outer = loop_heads ? head_stride : seq_stride, in_inner = loop_heads ? seq_stride : head_stride;
+    const long long sc_outer = loop_heads ? score_a : score_b, sc_inner = loop_heads ? score_b : score_a;
+    const long long ctx_outer = loop_heads ? (long long) d : (long long) S * H;
+    const long long ctx_inner = loop_heads ? (long long) S * H : (long long) d;
+
+    {
+    Timed t(profiler, Profiler::kAttentionGemm, stream);
+    for (int o = 0; o < outer; ++o) {
+        // column-major: scores_ba (S_k x S_q, ld S) = K_ba^T (d x S_k, ld 3H)^T * Q_ba (d x S_q, ld 3H)
+        cuBERT::blas_gemm_strided_batch(cublas, true, false, S, S, d, alpha, K + o * in_outer, ld, in_inner,
+                                        Q + o * in_outer, ld, in_inner, 0.f, attention_scores + o * sc_outer, S,
+                                        sc_inner, inner);
+    }
+    }
+    {
+        Timed t(profiler, Profiler::kMaskScaleSoftmax, stream);
+        cuBERT::mask_scale_softmax_(attention_scores, mask, 1.0f, B, A, S, stream);
+    }
+    Timed t(profiler, Profiler::kAttentionGemm, stream);
+    for (int o = 0; o < outer; ++o) {
+        // column-major: ctx_ba (d x S_q, ld H) = V_ba (d x S_k, ld 3H) * p_ba (S_k x S_q, ld S)
+        cuBERT::blas_gemm_strided_batch(cublas, false, false, d, S, S, 1.f, V + o * in_outer, ld, in_inner,
+                                        attention_scores + o * sc_outer, S, sc_inner, 0.f, context_out + o * ctx_outer,
+                                        H, ctx_inner, inner);
+    }
+}
+
+template <typename T>
+T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attention_mask) {
+    if (batch_size > max_batch_size) throw std::invalid_argument("batch_size > max_batch_size");
+    void *stream = cuBERT::blas_get_stream(cublas);
+    const int M = (int) (batch_size * seq_length), H = (int) hidden_size, I = (int) intermediate_size;
+
+    T *prev_output = input_gpu;
+    for (size_t l = 0; l < num_hidden_layers; ++l) {
+        const Layer &w = layers[l];
+        T *layer_input = prev_output;
+        T *out = layer_output[l & 1];
+
+        // attention/self: row-major Y[M, N] = X[M, K] W[K, N] is the column-major gemm(N, M, K) on (W, X)
+        {
+            Timed t(profiler, Profiler::kDenseGemm, stream);
+            cuBERT::blas_gemm(cublas, false, false, 3 * H, M, H, 1.f, w.qkv_kernel, 3 * H, layer_input, H, 0.f,
+                              qkv_out, 3 * H, w.qkv_bias);
+        }
+        attention(batch_size, qkv_out, attention_mask);
+
+        // attention/output: dense (bias deferred), then bias + residual(layer input) + LayerNorm
+        {
+            Timed t(profiler, Profiler::kDenseGemm, stream);
+            cuBERT::blas_gemm(cublas, false, false, H, M, H, 1.f, w.attention_output_kernel, H, context_out, H, 0.f,
+                              attention_output, H);
+        }
+        {
+            Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
+            cuBERT::layer_norm_(layer_input, attention_output, M, H, w.attention_output_bias, w.attention_norm_beta,
+                                w.attention_norm_gamma, stream);
+        }
+
+        // intermediate: dense (bias deferred), then bias + GELU
+        {
+            Timed t(profiler, Profiler::kDenseGemm, stream);
+            cuBERT::blas_gemm(cublas, false, false, I, M, H, 1.f, w.intermediate_kernel, I, attention_output, H, 0.f,
+                              intermediate_output, I);
+        }
+        {
+            Timed t(profiler, Profiler::kBiasGelu, stream);
+            cuBERT::gelu(intermediate_output, w.intermediate_bias, M, I, stream);
+        }
+
+        // output: dense (bias deferred), then bias + residual(attention output) + LayerNorm
+        {
+            Timed t(profiler, Profiler::kDenseGemm, stream);
+            cuBERT::blas_gemm(cublas, false, false, H, M, I, 1.f, w.output_kernel, H, intermediate_output, I, 0.f, out,
+                              H);
+        }
+        {
+            Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
+            cuBERT::layer_norm_(attention_output, out, M, H, w.output_bias, w.output_norm_beta, w.output_norm_gamma,
+                                stream);
+        }
+
+        prev_output = out;
+    }
+    return prev_output;
+}
+
+template class Transformer<float>;
+template class Transformer<half>;
+
+}  // namespace cuBERT

@@ -1,0 +1,83 @@
+// The encoder stack on one device.  Public surface of the reference's
+// Transformer<T> (src/cuBERT/op_att/Transformer.h:17-39): construct from the
+// named-weight map under a variable prefix, then compute(batch, input, mask)
+// with device pointers, returning a device pointer to [batch, seq, hidden].
+//
+// Inside, a layer is 6 GEMMs and 3 fused kernels:
+//   qkv   = x * [Wq|Wk|Wv] + [bq|bk|bv]          one GEMM, bias in its epilogue
+//   s     = (1/sqrt d) * Q K^T                    batched GEMM into scores[B, A, S, S]
+//   p     = softmax(s + mask)                     mask_scale_softmax_      (fused kernel)
+//   ctx   = p V                                   batched GEMM
+//   a     = LN(ctx * Wo + bo + x)                 GEMM, then layer_norm_   (fused kernel)
+//   i     = GELU(a * Wi + bi)                     GEMM, then gelu          (fused kernel)
+//   out   = LN(i * Wout + bout + a)               GEMM, then layer_norm_   (fused kernel)
+// Activation buffers are shared by all layers (the reference keeps four private
+// buffers per layer); weights live in one device allocation.
+#ifndef CUBERT_HOST_TRANSFORMER_H
+#define CUBERT_HOST_TRANSFORMER_H
+
+#include <cstddef>
+#include <cstdint>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "Arena.h"
+#include "Profiler.h"
+
+namespace cuBERT {
+
+template <typename T>
+class Transformer {
+public:
+    explicit Transformer(void *cublas, const std::string &var_prefix, const std::unordered_map<std::string, T *> &var,
+                         size_t max_batch_size, size_t seq_length, size_t hidden_size, size_t num_hidden_layers,
+                         size_t num_attention_heads, size_t intermediate_size);
+
+    virtual ~Transformer() = default;
+
+    T *compute(size_t batch_size, T *input_gpu, int8_t *attention_mask);
+
+    // Kept for source compatibility with callers of the reference: there the
+    // Dense outputs had to be pre-filled with their biases before a request;
+    // here biases are applied inside the GEMM epilogue or the fused kernels.
+    void _pre_compute(size_t batch_size);
+
+    T *_in_compute(size_t batch_size, T *input_gpu, int8_t *attention_mask);
+
+    // Optional per-kernel timing (owned by the caller; null = off).
+    void set_profiler(Profiler *p) { profiler = p; }
+
+private:
+    struct Layer {
+        T *qkv_kernel, *qkv_bias;            // [hidden, 3*hidden], [3*hidden]
+        T *attention_output_kernel, *attention_output_bias;
+        T *attention_norm_beta, *attention_norm_gamma;
+        T *intermediate_kernel, *intermediate_bias;
+        T *output_kernel, *output_bias;
+        T *output_norm_beta, *output_norm_gamma;
+    };
+
+    void layout_weights();
+    void layout_buffers();
+    void attention(size_t batch_size, const T *qkv, const int8_t *mask);
+
+    void *cublas;
+    Profiler *profiler = nullptr;
+    size_t max_batch_size, seq_length, hidden_size, num_hidden_layers, num_attention_heads, intermediate_size;
+
+    Arena weights;
+    Arena buffers;
+    std::vector<Layer> layers;
+
+    T *qkv_out;              // [M, 3*hidden]
+    T *attention_scores;     // [B, heads, seq, seq]
+    T *context_out;          // [M, hidden]
+    T *attention_output;     // [M, hidden]
+    T *intermediate_output;  // [M, intermediate]
+    T *layer_output[2];      // [M, hidden], alternating between layers
+};
+
+}  // namespace cuBERT
+
+#endif  // CUBERT_HOST_TRANSFORMER_H

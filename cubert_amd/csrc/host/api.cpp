@@ -1,0 +1,266 @@
+// The public C API (include/cuBERT.h) and the exception-free host entry points
+// (include/cubert_host.h).
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+
+#include "Bert.h"
+#include "BertM.h"
+#include "Transformer.h"
+#include "cuBERT.h"
+#include "cubert_host.h"
+
+using cuBERT::half;
+
+// ------------------------------------------------------------------ cuBERT.h
+
+void cuBERT_initialize() { cuBERT::initialize(); }
+
+void cuBERT_finalize() { cuBERT::finalize(); }
+
+int cuBERT_get_gpu_count() { return cuBERT::get_gpu_count(); }
+
+void *cuBERT_open(const char *model_file, int max_batch_size, int seq_length, int num_hidden_layers,
+                  int num_attention_heads, cuBERT_ComputeType compute_type) {
+    if (compute_type == cuBERT_COMPUTE_FLOAT) {
+        return new cuBERT::BertM<float>(model_file, max_batch_size, seq_length, num_hidden_layers, num_attention_heads);
+    }
+    return new cuBERT::BertM<half>(model_file, max_batch_size, seq_length, num_hidden_layers, num_attention_heads);
+}
+
+void cuBERT_compute(void *model, int batch_size, int *input_ids, int8_t *input_mask, int8_t *segment_ids, void *output,
+                    cuBERT_OutputType output_type, cuBERT_ComputeType compute_type) {
+    if (compute_type == cuBERT_COMPUTE_FLOAT) {
+        ((cuBERT::BertM<float> *) model)->compute(batch_size, input_ids, input_mask, segment_ids, (float *) output,
+                                                  output_type);
+    } else {
+        ((cuBERT::BertM<half> *) model)->compute(batch_size, input_ids, input_mask, segment_ids, (half *) output,
+                                                 output_type);
+    }
+}
+
+void cuBERT_compute_m(void *model, int batch_size, int *input_ids, int8_t *input_mask, int8_t *segment_ids,
+                      cuBERT_Output *output, cuBERT_ComputeType compute_type, int output_to_float) {
+    if (compute_type == cuBERT_COMPUTE_FLOAT) {
+        ((cuBERT::BertM<float> *) model)->compute(batch_size, input_ids, input_mask, segment_ids, output,
+                                                  output_to_float != 0);
+    } else {
+        ((cuBERT::BertM<half> *) model)->compute(batch_size, input_ids, input_mask, segment_ids, output,
+                                                 output_to_float != 0);
+    }
+}
+
+void cuBERT_close(void *model, cuBERT_ComputeType compute_type) {
+    if (compute_type == cuBERT_COMPUTE_FLOAT) {
+        delete (cuBERT::BertM<float> *) model;
+    } else {
+        delete (cuBERT::BertM<half> *) model;
+    }
+}
+
+// The WordPiece tokenizer is host-side string processing outside the device path this library
+// replaces; the symbols exist so that binaries linked against the reference still resolve.
+void *cuBERT_open_tokenizer(const char *, int) {
+    throw std::invalid_argument("tokenizer is not part of this build: tokenize on the host and call cuBERT_compute");
+}
+
+void cuBERT_close_tokenizer(void *) {}
+
+void cuBERT_tokenize_compute(void *, void *, int, const char **, const char **, void *, cuBERT_OutputType,
+                             cuBERT_ComputeType) {
+    throw std::invalid_argument("tokenizer is not part of this build: tokenize on the host and call cuBERT_compute");
+}
+
+void cuBERT_tokenize_compute_m(void *, void *, int, const char **, const char **, cuBERT_Output *, cuBERT_ComputeType,
+                               int) {
+    throw std::invalid_argument("tokenizer is not part of this build: tokenize on the host and call cuBERT_compute_m");
+}
+
+// ------------------------------------------------------------- cubert_host.h
+
+namespace {
+
+thread_local std::string g_last_error;
+
+template <typename F>
+int guarded(F &&f) {
+    try {
+        g_last_error.clear();
+        f();
+        return 0;
+    } catch (const std::invalid_argument &e) {
+        g_last_error = e.what();
+        return CUBERT_E_INVALID_ARGUMENT;
+    } catch (const std::out_of_range &e) {
+        g_last_error = e.what();
+        return CUBERT_E_OUT_OF_RANGE;
+    } catch (const std::exception &e) {
+        g_last_error = e.what();
+        return CUBERT_E_OTHER;
+    }
+}
+
+template <typename T>
+std::unordered_map<std::string, T *> var_map(int n, const char *const *names, const void *const *data) {
+    std::unordered_map<std::string, T *> var;
+    for (int i = 0; i < n; ++i) var[names[i]] = (T *) data[i];
+    return var;
+}
+
+template <typename T>
+void transformer_run(const char *prefix, int n, const char *const *names, const void *const *data, int batch, int seq,
+                     int hidden, int layers, int heads, int intermediate, const void *input, const int8_t *mask,
+                     void *output) {
+    void *stream = cuBERT::cuda_stream_create();
+    void *blas = cuBERT::blas_create();
+    cuBERT::blas_set_stream(blas, stream);
+    {
+        cuBERT::Transformer<T> transformer(blas, prefix, var_map<T>(n, names, data), batch, seq, hidden, layers, heads,
+                                           intermediate);
+        const size_t count = (size_t) batch * seq * hidden;
+        T *in_gpu = (T *) cuBERT::malloc(count * sizeof(T));
+        int8_t *mask_gpu = (int8_t *) cuBERT::malloc((size_t) batch * seq);
+        cuBERT::memcpy(in_gpu, input, count * sizeof(T), 1);
+        cuBERT::memcpy(mask_gpu, mask, (size_t) batch * seq, 1);
+        T *out_gpu = transformer.compute(batch, in_gpu, mask_gpu);
+        cuBERT::memcpyAsync(output, out_gpu, count * sizeof(T), 2, stream);
+        cuBERT::cuda_stream_synchronize(stream);
+        cuBERT::free(mask_gpu);
+        cuBERT::free(in_gpu);
+    }
+    cuBERT::blas_destroy(blas);
+    cuBERT::cuda_stream_destroy(stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *cubert_last_error(void) { return g_last_error.c_str(); }
+
+int cubert_try_open(const char *model_file, int max_batch_size, int seq_length, int num_hidden_layers,
+                    int num_attention_heads, int compute_type, void **model) {
+    return guarded([&] {
+        *model = cuBERT_open(model_file, max_batch_size, seq_length, num_hidden_layers, num_attention_heads,
+                             (cuBERT_ComputeType) compute_type);
+    });
+}
+
+int cubert_try_compute(void *model, int batch_size, int *input_ids, int8_t *input_mask, int8_t *segment_ids,
+                       void *output, int output_type, int compute_type) {
+    return guarded([&] {
+        cuBERT_compute(model, batch_size, input_ids, input_mask, segment_ids, output, (cuBERT_OutputType) output_type,
+                       (cuBERT_ComputeType) compute_type);
+    });
+}
+
+int cubert_try_compute_m(void *model, int batch_size, int *input_ids, int8_t *input_mask, int8_t *segment_ids,
+                         cuBERT_Output *output, int compute_type, int output_to_float) {
+    return guarded([&] {
+        cuBERT_compute_m(model, batch_size, input_ids, input_mask, segment_ids, output,
+                         (cuBERT_ComputeType) compute_type, output_to_float);
+    });
+}
+
+int cubert_try_close(void *model, int compute_type) {
+    return guarded([&] { cuBERT_close(model, (cuBERT_ComputeType) compute_type); });
+}
+
+int cubert_model_info(void *model, int compute_type, int *hidden_size, int *num_labels, int *seq_length) {
+    return guarded([&] {
+        if (model == nullptr) throw std::invalid_argument("null model");
+        if (compute_type == cuBERT_COMPUTE_FLOAT) {
+            auto *m = (cuBERT::BertM<float> *) model;
+            *hidden_size = (int) m->hidden_size(), *num_labels = (int) m->num_labels(), *seq_length = (int) m->seq_length;
+        } else {
+            auto *m = (cuBERT::BertM<half> *) model;
+            *hidden_size = (int) m->hidden_size(), *num_labels = (int) m->num_labels(), *seq_length = (int) m->seq_length;
+        }
+    });
+}
+
+int cubert_bert_create(int dtype, int n_vars, const char *const *names, const void *const *data, int max_batch_size,
+                       int seq_length, int vocab_size, int type_vocab_size, int hidden_size, int num_hidden_layers,
+                       int num_attention_heads, int intermediate_size, int num_labels, void **bert) {
+    return guarded([&] {
+        if (dtype == 0) {
+            *bert = new cuBERT::Bert<float>(var_map<float>(n_vars, names, data), max_batch_size, seq_length, vocab_size,
+                                            type_vocab_size, hidden_size, num_hidden_layers, num_attention_heads,
+                                            intermediate_size, num_labels);
+        } else {
+            *bert = new cuBERT::Bert<half>(var_map<half>(n_vars, names, data), max_batch_size, seq_length, vocab_size,
+                                           type_vocab_size, hidden_size, num_hidden_layers, num_attention_heads,
+                                           intermediate_size, num_labels);
+        }
+    });
+}
+
+int cubert_bert_compute(void *bert, int dtype, int batch_size, int *input_ids, int8_t *input_mask,
+                        int8_t *segment_ids) {
+    return guarded([&] {
+        if (dtype == 0) ((cuBERT::Bert<float> *) bert)->compute(batch_size, input_ids, input_mask, segment_ids);
+        else ((cuBERT::Bert<half> *) bert)->compute(batch_size, input_ids, input_mask, segment_ids);
+    });
+}
+
+int cubert_bert_output(void *bert, int dtype, int batch_size, cuBERT_Output *output, int output_to_float) {
+    return guarded([&] {
+        if (dtype == 0) {
+            ((cuBERT::Bert<float> *) bert)->output(batch_size, output);
+        } else if (output_to_float) {
+            ((cuBERT::Bert<half> *) bert)->output_to_float(batch_size, output);
+        } else {
+            ((cuBERT::Bert<half> *) bert)->output(batch_size, output);
+        }
+    });
+}
+
+int cubert_bert_compute_resident(void *bert, int dtype, int batch_size) {
+    return guarded([&] {
+        if (dtype == 0) ((cuBERT::Bert<float> *) bert)->compute_resident(batch_size);
+        else ((cuBERT::Bert<half> *) bert)->compute_resident(batch_size);
+    });
+}
+
+int cubert_bert_profile(void *bert, int dtype, unsigned kinds) {
+    return guarded([&] {
+        if (dtype == 0) ((cuBERT::Bert<float> *) bert)->profile(kinds);
+        else ((cuBERT::Bert<half> *) bert)->profile(kinds);
+    });
+}
+
+int cubert_bert_profile_read(void *bert, int dtype, double *total_ms, int *count, int n_kinds) {
+    return guarded([&] {
+        if (n_kinds < (int) cuBERT::Profiler::kKinds) throw std::invalid_argument("n_kinds too small");
+        if (dtype == 0) ((cuBERT::Bert<float> *) bert)->profile_read(total_ms, count);
+        else ((cuBERT::Bert<half> *) bert)->profile_read(total_ms, count);
+    });
+}
+
+void *cubert_bert_stream(void *bert, int dtype) {
+    return dtype == 0 ? ((cuBERT::Bert<float> *) bert)->get_stream() : ((cuBERT::Bert<half> *) bert)->get_stream();
+}
+
+int cubert_bert_destroy(void *bert, int dtype) {
+    return guarded([&] {
+        if (dtype == 0) delete (cuBERT::Bert<float> *) bert;
+        else delete (cuBERT::Bert<half> *) bert;
+    });
+}
+
+int cubert_transformer_run(int dtype, const char *var_prefix, int n_vars, const char *const *names,
+                           const void *const *data, int batch_size, int seq_length, int hidden_size,
+                           int num_hidden_layers, int num_attention_heads, int intermediate_size, const void *input,
+                           const int8_t *mask, void *output) {
+    return guarded([&] {
+        if (dtype == 0) {
+            transformer_run<float>(var_prefix, n_vars, names, data, batch_size, seq_length, hidden_size,
+                                   num_hidden_layers, num_attention_heads, intermediate_size, input, mask, output);
+        } else {
+            transformer_run<half>(var_prefix, n_vars, names, data, batch_size, seq_length, hidden_size,
+                                  num_hidden_layers, num_attention_heads, intermediate_size, input, mask, output);
+        }
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,97 @@
+// Shared device helpers for the gfx950 layer kernels: 16-byte vector access,
+// storage <-> fp32 conversion and cross-lane reductions for 64-wide wavefronts.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace cubert {
+
+constexpr int kWave = 64;        // CDNA wavefront width
+constexpr int kBlock = 256;      // threads per workgroup used by every kernel here (4 wavefronts)
+
+typedef _Float16 half_t;         // IEEE binary16 storage type
+
+// N consecutive elements moved with one memory instruction (N * sizeof(T) <= 16 bytes).
+template <typename T, int N>
+struct alignas(sizeof(T) * N) Vec {
+    T v[N];
+};
+
+template <typename T, int N>
+__device__ __forceinline__ Vec<T, N> load_vec(const T *p) {
+    return *reinterpret_cast<const Vec<T, N> *>(p);
+}
+
+template <typename T, int N>
+__device__ __forceinline__ void store_vec(T *p, const Vec<T, N> &x) {
+    *reinterpret_cast<Vec<T, N> *>(p) = x;
+}
+
+__device__ __forceinline__ float to_f32(float x) { return x; }
+__device__ __forceinline__ float to_f32(half_t x) { return (float) x; }
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float x);
+template <>
+__device__ __forceinline__ float from_f32<float>(float x) { return x; }
+template <>
+__device__ __forceinline__ half_t from_f32<half_t>(float x) { return (half_t) x; }  // round to nearest even
+
+// Widest vector (in elements) that is at most 16 bytes.
+template <typename T>
+struct MaxVec {
+    static constexpr int value = 16 / sizeof(T);
+};
+
+// ---- cross-lane exchange -------------------------------------------------
+// DPP moves data between lanes of a row of 16 in the same instruction slot as
+// an ALU op; 32- and 64-lane steps go through the LDS crossbar (ds_bpermute).
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    int i = __builtin_bit_cast(int, v);
+    i = __builtin_amdgcn_update_dpp(i, i, CTRL, 0xf, 0xf, false);
+    return __builtin_bit_cast(float, i);
+}
+
+constexpr int kDppQuadXor1 = 0xB1;       // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;       // quad_perm:[2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141; // lane i <- lane 7-i within each 8 lanes
+constexpr int kDppRowMirror = 0x140;     // lane i <- lane 15-i within each 16 lanes
+
+struct SumOp {
+    __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+struct MaxOp {
+    __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+};
+
+// All-reduce over aligned groups of LANES consecutive lanes (LANES = 1..64, a
+// power of two).  Every lane of a group ends up with the group's result.
+template <int LANES, typename Op>
+__device__ __forceinline__ float group_reduce(float v, Op op) {
+    static_assert(LANES >= 1 && LANES <= 64 && (LANES & (LANES - 1)) == 0, "LANES must be a power of two");
+    if (LANES >= 2) v = op(v, dpp_move<kDppQuadXor1>(v));
+    if (LANES >= 4) v = op(v, dpp_move<kDppQuadXor2>(v));
+    if (LANES >= 8) v = op(v, dpp_move<kDppRowHalfMirror>(v));
+    if (LANES >= 16) v = op(v, dpp_move<kDppRowMirror>(v));
+    if (LANES >= 32) v = op(v, __shfl_xor(v, 16, kWave));
+    if (LANES >= 64) v = op(v, __shfl_xor(v, 32, kWave));
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) { return group_reduce<kWave>(v, SumOp()); }
+__device__ __forceinline__ float wave_max(float v) { return group_reduce<kWave>(v, MaxOp()); }
+
+// Wavefront index inside the workgroup as a scalar (SGPR) value, so that
+// addresses derived from it use scalar arithmetic and scalar loads.
+__device__ __forceinline__ int wave_in_block() {
+    return __builtin_amdgcn_readfirstlane((int) (threadIdx.x >> 6));
+}
+
+__host__ __device__ __forceinline__ bool is_aligned(const void *p, size_t bytes) {
+    return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0;
+}
+
+}  // namespace cubert

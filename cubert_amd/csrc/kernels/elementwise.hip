@@ -1,0 +1,212 @@
+// Streaming kernels: bias + GELU, bias + tanh, mean over the sequence axis and
+// the plain embedding-row gather.  All are one read + one write per element
+// with 16-byte accesses; arithmetic in fp32.
+
+#include "cubert_kernels.h"
+#include "device_common.h"
+
+namespace cubert {
+namespace {
+
+inline int launch_status() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : (int) e;
+}
+
+struct GeluOp {
+    // reference: op/GELU.cpp:13 -- x * 0.5f * (1.0f + erff(x * sqrtf(0.5f)))
+    __device__ __forceinline__ float operator()(float x) const { return x * 0.5f * (1.0f + erff(x * 0.70710678118654752440f)); }
+};
+struct TanhOp {
+    // reference: op_bert/BertPooler.cpp:13
+    __device__ __forceinline__ float operator()(float x) const { return tanhf(x); }
+};
+
+// [rows, width] in place, y = f(x + bias[col]).  A workgroup owns ROWS
+// consecutive rows; its threads walk the columns, so the bias vector of a
+// column is loaded once and reused for the ROWS rows, and no index division is
+// needed.  width must be a multiple of VEC.
+template <typename T, typename Op, int VEC, int ROWS>
+__global__ __launch_bounds__(kBlock) void bias_act_kernel(T *__restrict__ inout, const T *__restrict__ bias, int rows,
+                                                          int width) {
+    const int row0 = blockIdx.x * ROWS;
+    Op op;
+    for (int col = threadIdx.x * VEC; col < width; col += blockDim.x * VEC) {
+        float b[VEC];
+        if (bias != nullptr) {
+            Vec<T, VEC> bv = load_vec<T, VEC>(bias + col);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) b[i] = to_f32(bv.v[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) b[i] = 0.f;
+        }
+        Vec<T, VEC> x[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            if (row0 + r < rows) x[r] = load_vec<T, VEC>(inout + (size_t) (row0 + r) * width + col);
+        }
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            if (row0 + r < rows) {
+                Vec<T, VEC> y;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) y.v[i] = from_f32<T>(op(to_f32(x[r].v[i]) + b[i]));
+                store_vec<T, VEC>(inout + (size_t) (row0 + r) * width + col, y);
+            }
+        }
+    }
+}
+
+// Threads per workgroup so that the column walk has no ragged last trip when possible.
+inline int pick_threads(int vectors_per_row) {
+    for (int t = kBlock; t >= kWave; t -= kWave) {
+        if (vectors_per_row % t == 0) return t;
+    }
+    return vectors_per_row < kBlock ? ((vectors_per_row + kWave - 1) / kWave) * kWave : kBlock;
+}
+
+template <typename T, typename Op>
+int bias_act(T *inout, const T *bias, int rows, int width, void *stream) {
+    if (rows < 0 || width <= 0 || !inout) return CUBERT_BAD_ARGUMENT;
+    if (rows == 0) return 0;
+    hipStream_t s = (hipStream_t) stream;
+    constexpr int V = MaxVec<T>::value;
+    if (width % V == 0 && is_aligned(inout, 16) && (bias == nullptr || is_aligned(bias, 16))) {
+        const int threads = pick_threads(width / V);
+        // Many rows: 4 per workgroup (deeper load queue); few rows: 1 per workgroup (more workgroups).
+        if ((long long) rows * width * (long long) sizeof(T) >= (16LL << 20)) {
+            hipLaunchKernelGGL((bias_act_kernel<T, Op, V, 4>), dim3((rows + 3) / 4), dim3(threads), 0, s, inout, bias,
+                               rows, width);
+        } else {
+            hipLaunchKernelGGL((bias_act_kernel<T, Op, V, 1>), dim3(rows), dim3(threads), 0, s, inout, bias, rows,
+                               width);
+        }
+    } else {
+        hipLaunchKernelGGL((bias_act_kernel<T, Op, 1, 1>), dim3(rows), dim3(kBlock), 0, s, inout, bias, rows, width);
+    }
+    return launch_status();
+}
+
+// out[b, c] = mean_s in[b, s, c].  grid = (column tiles, batch); the block's
+// wavefronts split the sequence, each lane keeps VEC channel sums, and the
+// partial sums meet in LDS.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void mean_pool_kernel(const T *__restrict__ in, T *__restrict__ out, int seq,
+                                                           int hidden) {
+    __shared__ float partial[kBlock / kWave][kWave * VEC];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = wave_in_block();
+    const int col = (blockIdx.x * kWave + lane) * VEC;
+    const int b = blockIdx.y;
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+    if (col < hidden) {
+        const T *p = in + (size_t) b * seq * hidden + col;
+        for (int s = wave; s < seq; s += kBlock / kWave) {
+            Vec<T, VEC> v = load_vec<T, VEC>(p + (size_t) s * hidden);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] += to_f32(v.v[i]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) partial[wave][lane * VEC + i] = acc[i];
+    __syncthreads();
+    if (wave == 0 && col < hidden) {
+        Vec<T, VEC> o;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            float t = partial[0][lane * VEC + i];
+#pragma unroll
+            for (int w = 1; w < kBlock / kWave; ++w) t += partial[w][lane * VEC + i];
+            o.v[i] = from_f32<T>(t / (float) seq);
+        }
+        store_vec<T, VEC>(out + (size_t) b * hidden + col, o);
+    }
+}
+
+template <typename T>
+int mean_pool(const T *in, T *out, int batch, int seq, int hidden, void *stream) {
+    if (batch < 0 || seq <= 0 || hidden <= 0 || !in || !out || batch > 65535) return CUBERT_BAD_ARGUMENT;
+    if (batch == 0) return 0;
+    hipStream_t s = (hipStream_t) stream;
+    constexpr int V = MaxVec<T>::value;
+    if (hidden % V == 0 && is_aligned(in, 16) && is_aligned(out, 16)) {
+        dim3 grid((hidden / V + kWave - 1) / kWave, batch);
+        hipLaunchKernelGGL((mean_pool_kernel<T, V>), grid, dim3(kBlock), 0, s, in, out, seq, hidden);
+    } else {
+        dim3 grid((hidden + kWave - 1) / kWave, batch);
+        hipLaunchKernelGGL((mean_pool_kernel<T, 1>), grid, dim3(kBlock), 0, s, in, out, seq, hidden);
+    }
+    return launch_status();
+}
+
+// out[i, :] = table[ids[i], :]; one wavefront per row.
+template <typename T, typename Id, int VEC>
+__global__ __launch_bounds__(kBlock) void gather_kernel(const Id *__restrict__ ids, int n, const T *__restrict__ table,
+                                                        int width, T *__restrict__ out) {
+    const int row = blockIdx.x * (kBlock / kWave) + wave_in_block();
+    if (row >= n) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const T *src = table + (size_t) ids[row] * width;
+    T *dst = out + (size_t) row * width;
+    for (int col = lane * VEC; col < width; col += kWave * VEC) {
+        store_vec<T, VEC>(dst + col, load_vec<T, VEC>(src + col));
+    }
+}
+
+template <typename T, typename Id>
+int gather(const Id *ids, int n, const T *table, int width, T *out, void *stream) {
+    if (n < 0 || width <= 0 || !ids || !table || !out) return CUBERT_BAD_ARGUMENT;
+    if (n == 0) return 0;
+    hipStream_t s = (hipStream_t) stream;
+    constexpr int V = MaxVec<T>::value;
+    dim3 grid((n + 3) / 4), block(kBlock);
+    if (width % V == 0 && is_aligned(table, 16) && is_aligned(out, 16)) {
+        hipLaunchKernelGGL((gather_kernel<T, Id, V>), grid, block, 0, s, ids, n, table, width, out);
+    } else {
+        hipLaunchKernelGGL((gather_kernel<T, Id, 1>), grid, block, 0, s, ids, n, table, width, out);
+    }
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace cubert
+
+using cubert::half_t;
+
+extern "C" int cubert_bias_gelu_f32(float *inout, const float *bias, int rows, int width, void *stream) {
+    return cubert::bias_act<float, cubert::GeluOp>(inout, bias, rows, width, stream);
+}
+extern "C" int cubert_bias_gelu_f16(cubert_half *inout, const cubert_half *bias, int rows, int width, void *stream) {
+    return cubert::bias_act<half_t, cubert::GeluOp>((half_t *) inout, (const half_t *) bias, rows, width, stream);
+}
+extern "C" int cubert_bias_tanh_f32(float *inout, const float *bias, int rows, int width, void *stream) {
+    return cubert::bias_act<float, cubert::TanhOp>(inout, bias, rows, width, stream);
+}
+extern "C" int cubert_bias_tanh_f16(cubert_half *inout, const cubert_half *bias, int rows, int width, void *stream) {
+    return cubert::bias_act<half_t, cubert::TanhOp>((half_t *) inout, (const half_t *) bias, rows, width, stream);
+}
+extern "C" int cubert_mean_pool_f32(const float *in, float *out, int batch, int seq_length, int hidden, void *stream) {
+    return cubert::mean_pool<float>(in, out, batch, seq_length, hidden, stream);
+}
+extern "C" int cubert_mean_pool_f16(const cubert_half *in, cubert_half *out, int batch, int seq_length, int hidden,
+                                    void *stream) {
+    return cubert::mean_pool<half_t>((const half_t *) in, (half_t *) out, batch, seq_length, hidden, stream);
+}
+extern "C" int cubert_gather_f32(const int32_t *ids, int n, const float *table, int width, float *out, void *stream) {
+    return cubert::gather<float, int32_t>(ids, n, table, width, out, stream);
+}
+extern "C" int cubert_gather_f16(const int32_t *ids, int n, const cubert_half *table, int width, cubert_half *out,
+                                 void *stream) {
+    return cubert::gather<half_t, int32_t>(ids, n, (const half_t *) table, width, (half_t *) out, stream);
+}
+extern "C" int cubert_gather_i8_f32(const int8_t *ids, int n, const float *table, int width, float *out,
+                                    void *stream) {
+    return cubert::gather<float, int8_t>(ids, n, table, width, out, stream);
+}
+extern "C" int cubert_gather_i8_f16(const int8_t *ids, int n, const cubert_half *table, int width, cubert_half *out,
+                                    void *stream) {
+    return cubert::gather<half_t, int8_t>(ids, n, (const half_t *) table, width, (half_t *) out, stream);
+}

@@ -1,0 +1,303 @@
+// Row kernels that end in a LayerNorm: embedding gather + LayerNorm and
+// bias + residual + LayerNorm.  One 64-lane wavefront owns one row of `hidden`
+// elements; the row lives in registers between the statistics pass and the
+// normalisation, so HBM sees each operand once (2 reads + 1 write per element
+// for bias_res_ln, 1 gathered read + 1 write for embed_ln).
+//
+// Arithmetic follows the reference's CPU code (op/LayerNorm.cpp:20-41):
+// sums of x and x*x in fp32, biased variance E[x^2] - mean^2, epsilon 1e-12
+// inside the square root, out = beta + gamma * rstd * (x - mean).  The sums are
+// tree-reduced across lanes instead of accumulated serially.  A variance that
+// cancellation drives below zero is clamped to zero (the reference would take
+// the square root of a negative number there).
+
+#include <initializer_list>
+
+#include "cubert_kernels.h"
+#include "device_common.h"
+
+namespace cubert {
+namespace {
+
+constexpr int kRowsPerBlock = kBlock / kWave;  // 4
+
+__device__ __forceinline__ void ln_stats(float sum, float sumsq, int hidden, float &mean, float &rstd) {
+    sum = wave_sum(sum);
+    sumsq = wave_sum(sumsq);
+    mean = sum / (float) hidden;
+    float var = sumsq / (float) hidden - mean * mean;
+    var = fmaxf(var, 0.f);
+    rstd = 1.f / sqrtf(var + 1e-12f);
+}
+
+// ---- fast path: hidden == 64 * VEC * CHUNKS, everything 16-byte friendly ----
+
+// Normalise the row held in x[][] and store it.  gamma/beta were loaded before
+// the reduction so their latency overlaps it.
+template <typename T, int VEC, int CHUNKS>
+__device__ __forceinline__ void ln_finish(float (&x)[CHUNKS][VEC], float sum, float sumsq, const Vec<T, VEC> (&g)[CHUNKS],
+                                          const Vec<T, VEC> (&b)[CHUNKS], T *__restrict__ out_row, int lane) {
+    float mean, rstd;
+    ln_stats(sum, sumsq, kWave * VEC * CHUNKS, mean, rstd);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        Vec<T, VEC> o;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            o.v[i] = from_f32<T>(to_f32(b[c].v[i]) + (to_f32(g[c].v[i]) * rstd) * (x[c][i] - mean));
+        }
+        store_vec<T, VEC>(out_row + (c * kWave + lane) * VEC, o);
+    }
+}
+
+template <typename T, int VEC, int CHUNKS, bool HAS_BIAS>
+__global__ __launch_bounds__(kBlock) void bias_res_ln_kernel(T *__restrict__ inout, const T *__restrict__ residual,
+                                                             const T *__restrict__ bias, const T *__restrict__ beta,
+                                                             const T *__restrict__ gamma, int rows) {
+    constexpr int H = kWave * VEC * CHUNKS;
+    const int row = blockIdx.x * kRowsPerBlock + wave_in_block();
+    if (row >= rows) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    T *io = inout + (size_t) row * H;
+    const T *res = residual + (size_t) row * H;
+
+    // every load of the row is issued before the first use
+    Vec<T, VEC> a[CHUNKS], r[CHUNKS], bi[CHUNKS], g[CHUNKS], be[CHUNKS];
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int col = (c * kWave + lane) * VEC;
+        a[c] = load_vec<T, VEC>(io + col);
+        r[c] = load_vec<T, VEC>(res + col);
+    }
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int col = (c * kWave + lane) * VEC;
+        if (HAS_BIAS) bi[c] = load_vec<T, VEC>(bias + col);
+        g[c] = load_vec<T, VEC>(gamma + col);
+        be[c] = load_vec<T, VEC>(beta + col);
+    }
+    float x[CHUNKS][VEC];
+    float sum = 0.f, sumsq = 0.f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            // (gemm output + bias) + residual: the order the reference adds them in
+            float v = to_f32(a[c].v[i]);
+            if (HAS_BIAS) v += to_f32(bi[c].v[i]);
+            v += to_f32(r[c].v[i]);
+            x[c][i] = v;
+            sum += v;
+            sumsq += v * v;
+        }
+    }
+    ln_finish<T, VEC, CHUNKS>(x, sum, sumsq, g, be, io, lane);
+}
+
+template <typename T, int VEC, int CHUNKS>
+__global__ __launch_bounds__(kBlock) void embed_ln_kernel(const int32_t *__restrict__ ids,
+                                                          const int8_t *__restrict__ segments,
+                                                          const T *__restrict__ word, const T *__restrict__ pos,
+                                                          const T *__restrict__ type, const T *__restrict__ beta,
+                                                          const T *__restrict__ gamma, T *__restrict__ out, int rows,
+                                                          int seq_length) {
+    constexpr int H = kWave * VEC * CHUNKS;
+    const int row = blockIdx.x * kRowsPerBlock + wave_in_block();
+    if (row >= rows) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    // row is wavefront-uniform, so these are scalar loads
+    const T *w = word + (size_t) ids[row] * H;
+    const T *t = type + (size_t) segments[row] * H;
+    const T *p = pos + (size_t) (row % seq_length) * H;
+
+    Vec<T, VEC> a[CHUNKS], b[CHUNKS], d[CHUNKS], g[CHUNKS], be[CHUNKS];
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int col = (c * kWave + lane) * VEC;
+        a[c] = load_vec<T, VEC>(w + col);
+        b[c] = load_vec<T, VEC>(p + col);
+        d[c] = load_vec<T, VEC>(t + col);
+    }
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int col = (c * kWave + lane) * VEC;
+        g[c] = load_vec<T, VEC>(gamma + col);
+        be[c] = load_vec<T, VEC>(beta + col);
+    }
+    float x[CHUNKS][VEC];
+    float sum = 0.f, sumsq = 0.f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            // (word + position) + token type: the order the reference adds them in
+            float v = (to_f32(a[c].v[i]) + to_f32(b[c].v[i])) + to_f32(d[c].v[i]);
+            x[c][i] = v;
+            sum += v;
+            sumsq += v * v;
+        }
+    }
+    ln_finish<T, VEC, CHUNKS>(x, sum, sumsq, g, be, out + (size_t) row * H, lane);
+}
+
+// ---- generic path: any hidden size, scalar accesses, operands read twice ----
+
+template <typename T, bool EMBED>
+__global__ __launch_bounds__(kBlock) void ln_generic_kernel(T *__restrict__ inout, const T *__restrict__ residual,
+                                                            const T *__restrict__ bias,
+                                                            const int32_t *__restrict__ ids,
+                                                            const int8_t *__restrict__ segments,
+                                                            const T *__restrict__ word, const T *__restrict__ pos,
+                                                            const T *__restrict__ type, const T *__restrict__ beta,
+                                                            const T *__restrict__ gamma, int rows, int hidden,
+                                                            int seq_length) {
+    const int row = blockIdx.x * kRowsPerBlock + wave_in_block();
+    if (row >= rows) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const T *a, *b, *c;
+    if (EMBED) {
+        a = word + (size_t) ids[row] * hidden;
+        b = pos + (size_t) (row % seq_length) * hidden;
+        c = type + (size_t) segments[row] * hidden;
+    } else {
+        a = inout + (size_t) row * hidden;
+        b = bias;  // may be null
+        c = residual + (size_t) row * hidden;
+    }
+    T *o = inout + (size_t) row * hidden;
+
+    float sum = 0.f, sumsq = 0.f;
+    for (int j = lane; j < hidden; j += kWave) {
+        float x = to_f32(a[j]);
+        if (EMBED || b != nullptr) x += to_f32(b[j]);
+        x += to_f32(c[j]);
+        sum += x;
+        sumsq += x * x;
+    }
+    float mean, rstd;
+    ln_stats(sum, sumsq, hidden, mean, rstd);
+    for (int j = lane; j < hidden; j += kWave) {
+        float x = to_f32(a[j]);
+        if (EMBED || b != nullptr) x += to_f32(b[j]);
+        x += to_f32(c[j]);
+        o[j] = from_f32<T>(to_f32(beta[j]) + (to_f32(gamma[j]) * rstd) * (x - mean));
+    }
+}
+
+inline int launch_status() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : (int) e;
+}
+
+template <typename T>
+bool vector_ok(int hidden, int vec, std::initializer_list<const void *> ptrs) {
+    if (hidden % (kWave * vec) != 0) return false;
+    for (const void *p : ptrs) {
+        if (p != nullptr && !is_aligned(p, sizeof(T) * vec)) return false;
+    }
+    return true;
+}
+
+template <typename T>
+int bias_res_ln(T *inout, const T *residual, const T *bias, const T *beta, const T *gamma, int rows, int hidden,
+                void *stream) {
+    if (rows < 0 || hidden <= 0 || !inout || !residual || !beta || !gamma) return CUBERT_BAD_ARGUMENT;
+    if (rows == 0) return 0;
+    hipStream_t s = (hipStream_t) stream;
+    dim3 grid((rows + kRowsPerBlock - 1) / kRowsPerBlock), block(kBlock);
+    constexpr int V = MaxVec<T>::value;  // 4 floats or 8 halves
+#define CUBERT_LN_CASE(VEC, CHUNKS)                                                                      \
+    if (hidden == kWave * VEC * CHUNKS && vector_ok<T>(hidden, VEC, {inout, residual, bias, beta, gamma})) { \
+        if (bias != nullptr)                                                                             \
+            hipLaunchKernelGGL((bias_res_ln_kernel<T, VEC, CHUNKS, true>), grid, block, 0, s, inout, residual, bias, \
+                               beta, gamma, rows);                                                       \
+        else                                                                                             \
+            hipLaunchKernelGGL((bias_res_ln_kernel<T, VEC, CHUNKS, false>), grid, block, 0, s, inout, residual, bias, \
+                               beta, gamma, rows);                                                       \
+        return launch_status();                                                                          \
+    }
+    CUBERT_LN_CASE(V, 1)
+    CUBERT_LN_CASE(V, 2)
+    CUBERT_LN_CASE(V, 3)
+    CUBERT_LN_CASE(V, 4)
+    CUBERT_LN_CASE(V / 2, 1)
+    CUBERT_LN_CASE(V / 2, 3)  // 768 halves = 64 lanes x 4 x 3
+    CUBERT_LN_CASE(V / 2, 5)
+    CUBERT_LN_CASE(V / 2, 7)
+    CUBERT_LN_CASE(V, 5)
+    CUBERT_LN_CASE(V, 6)
+    CUBERT_LN_CASE(V, 8)
+#undef CUBERT_LN_CASE
+    hipLaunchKernelGGL((ln_generic_kernel<T, false>), grid, block, 0, s, inout, residual, bias, nullptr, nullptr,
+                       nullptr, nullptr, nullptr, beta, gamma, rows, hidden, 1);
+    return launch_status();
+}
+
+template <typename T>
+int embed_ln(const int32_t *ids, const int8_t *segments, const T *word, const T *pos, const T *type, const T *beta,
+             const T *gamma, T *out, int batch, int seq_length, int hidden, void *stream) {
+    if (batch < 0 || seq_length <= 0 || hidden <= 0 || !ids || !segments || !word || !pos || !type || !beta ||
+        !gamma || !out)
+        return CUBERT_BAD_ARGUMENT;
+    const long long rows_ll = (long long) batch * seq_length;
+    if (rows_ll > 0x7fffffffLL) return CUBERT_BAD_ARGUMENT;
+    const int rows = (int) rows_ll;
+    if (rows == 0) return 0;
+    hipStream_t s = (hipStream_t) stream;
+    dim3 grid((rows + kRowsPerBlock - 1) / kRowsPerBlock), block(kBlock);
+    constexpr int V = MaxVec<T>::value;
+#define CUBERT_EMB_CASE(VEC, CHUNKS)                                                                       \
+    if (hidden == kWave * VEC * CHUNKS && vector_ok<T>(hidden, VEC, {word, pos, type, beta, gamma, out})) { \
+        hipLaunchKernelGGL((embed_ln_kernel<T, VEC, CHUNKS>), grid, block, 0, s, ids, segments, word, pos, type, \
+                           beta, gamma, out, rows, seq_length);                                            \
+        return launch_status();                                                                            \
+    }
+    CUBERT_EMB_CASE(V, 1)
+    CUBERT_EMB_CASE(V, 2)
+    CUBERT_EMB_CASE(V, 3)
+    CUBERT_EMB_CASE(V, 4)
+    CUBERT_EMB_CASE(V / 2, 1)
+    CUBERT_EMB_CASE(V / 2, 3)
+    CUBERT_EMB_CASE(V / 2, 5)
+    CUBERT_EMB_CASE(V / 2, 7)
+    CUBERT_EMB_CASE(V, 5)
+    CUBERT_EMB_CASE(V, 6)
+    CUBERT_EMB_CASE(V, 8)
+#undef CUBERT_EMB_CASE
+    hipLaunchKernelGGL((ln_generic_kernel<T, true>), grid, block, 0, s, out, nullptr, nullptr, ids, segments, word,
+                       pos, type, beta, gamma, rows, hidden, seq_length);
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace cubert
+
+using cubert::half_t;
+
+extern "C" int cubert_bias_res_ln_f32(float *inout, const float *residual, const float *bias, const float *beta,
+                                      const float *gamma, int rows, int hidden, void *stream) {
+    return cubert::bias_res_ln<float>(inout, residual, bias, beta, gamma, rows, hidden, stream);
+}
+
+extern "C" int cubert_bias_res_ln_f16(cubert_half *inout, const cubert_half *residual, const cubert_half *bias,
+                                      const cubert_half *beta, const cubert_half *gamma, int rows, int hidden,
+                                      void *stream) {
+    return cubert::bias_res_ln<half_t>((half_t *) inout, (const half_t *) residual, (const half_t *) bias,
+                                       (const half_t *) beta, (const half_t *) gamma, rows, hidden, stream);
+}
+
+extern "C" int cubert_embed_ln_f32(const int32_t *ids, const int8_t *segments, const float *word, const float *pos,
+                                   const float *type, const float *beta, const float *gamma, float *out, int batch,
+                                   int seq_length, int hidden, void *stream) {
+    return cubert::embed_ln<float>(ids, segments, word, pos, type, beta, gamma, out, batch, seq_length, hidden,
+                                   stream);
+}
+
+extern "C" int cubert_embed_ln_f16(const int32_t *ids, const int8_t *segments, const cubert_half *word,
+                                   const cubert_half *pos, const cubert_half *type, const cubert_half *beta,
+                                   const cubert_half *gamma, cubert_half *out, int batch, int seq_length, int hidden,
+                                   void *stream) {
+    return cubert::embed_ln<half_t>(ids, segments, (const half_t *) word, (const half_t *) pos,
+                                    (const half_t *) type, (const half_t *) beta, (const half_t *) gamma,
+                                    (half_t *) out, batch, seq_length, hidden, stream);
+}

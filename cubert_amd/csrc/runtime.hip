@@ -1,0 +1,359 @@
+// Device runtime of the library: memory, copies, streams and GEMM.
+// The only translation unit that talks to the HIP runtime API and hipBLASLt
+// (the layer kernels launch through hipLaunchKernelGGL in their own files).
+//
+// GEMMs use hipBLASLt with fp32 accumulation (HIPBLAS_COMPUTE_32F) for both
+// storage types; plans (descriptor + layouts + the algorithm the heuristic
+// ranks first) are cached per shape in the BLAS context, so a steady-state call
+// is one hipblasLtMatmul.
+
+#include <hip/hip_runtime.h>
+#include <hipblaslt/hipblaslt.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <map>
+#include <mutex>
+#include <string>
+#include <tuple>
+#include <vector>
+
+#include "cubert_kernels.h"
+
+namespace {
+
+inline int hip_rc(hipError_t e) { return e == hipSuccess ? 0 : (int) e; }
+
+hipMemcpyKind copy_kind(int kind) {
+    switch (kind) {
+        case 1: return hipMemcpyHostToDevice;
+        case 2: return hipMemcpyDeviceToHost;
+        case 3: return hipMemcpyDeviceToDevice;
+        case 0: return hipMemcpyHostToHost;
+        default: return hipMemcpyDefault;
+    }
+}
+
+constexpr size_t kWorkspaceBytes = 64u << 20;
+
+struct GemmKey {
+    int type;  // 0 = f32, 1 = f16
+    int transA, transB, M, N, K, lda, ldb, ldc, batch;
+    long long strideA, strideB, strideC;
+    bool bias;
+    bool beta_zero;
+    bool operator<(const GemmKey &o) const {
+        return std::tie(type, transA, transB, M, N, K, lda, ldb, ldc, batch, strideA, strideB, strideC, bias, beta_zero) <
+               std::tie(o.type, o.transA, o.transB, o.M, o.N, o.K, o.lda, o.ldb, o.ldc, o.batch, o.strideA, o.strideB,
+                        o.strideC, o.bias, o.beta_zero);
+    }
+};
+
+struct GemmPlan {
+    hipblasLtMatmulDesc_t desc = nullptr;
+    hipblasLtMatrixLayout_t a = nullptr, b = nullptr, c = nullptr;
+    hipblasLtMatmulAlgo_t algo;
+    size_t workspace = 0;
+    bool ok = false;  // false: hipBLASLt has no algorithm for this shape, the plain kernel runs instead
+};
+
+struct BlasContext {
+    hipblasLtHandle_t lt = nullptr;
+    hipStream_t stream = nullptr;
+    void *workspace = nullptr;
+    std::map<GemmKey, GemmPlan> plans;
+    std::mutex mutex;
+};
+
+#define LT_TRY(call)                                                                                      \
+    do {                                                                                                  \
+        hipblasStatus_t st_ = (call);                                                                     \
+        if (st_ != HIPBLAS_STATUS_SUCCESS) {                                                              \
+            fprintf(stderr, "hipBLASLt error %d at %s:%d: %s\n", (int) st_, __FILE__, __LINE__, #call);   \
+            return 1000 + (int) st_;                                                                      \
+        }                                                                                                 \
+    } while (0)
+
+int make_layout(hipblasLtMatrixLayout_t *out, hipDataType type, int rows, int cols, int ld, int batch,
+                long long stride) {
+    LT_TRY(hipblasLtMatrixLayoutCreate(out, type, (uint64_t) rows, (uint64_t) cols, (int64_t) ld));
+    if (batch > 1) {
+        int32_t bc = batch;
+        int64_t st = stride;
+        LT_TRY(hipblasLtMatrixLayoutSetAttribute(*out, HIPBLASLT_MATRIX_LAYOUT_BATCH_COUNT, &bc, sizeof bc));
+        LT_TRY(hipblasLtMatrixLayoutSetAttribute(*out, HIPBLASLT_MATRIX_LAYOUT_STRIDED_BATCH_OFFSET, &st, sizeof st));
+    }
+    return 0;
+}
+
+int build_plan(BlasContext *ctx, const GemmKey &k, GemmPlan *plan) {
+    const hipDataType type = k.type == 0 ? HIP_R_32F : HIP_R_16F;
+    LT_TRY(hipblasLtMatmulDescCreate(&plan->desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
+    hipblasOperation_t ta = k.transA ? HIPBLAS_OP_T : HIPBLAS_OP_N, tb = k.transB ? HIPBLAS_OP_T : HIPBLAS_OP_N;
+    LT_TRY(hipblasLtMatmulDescSetAttribute(plan->desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof ta));
+    LT_TRY(hipblasLtMatmulDescSetAttribute(plan->desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof tb));
+    if (k.bias) {
+        hipblasLtEpilogue_t ep = HIPBLASLT_EPILOGUE_BIAS;
+        LT_TRY(hipblasLtMatmulDescSetAttribute(plan->desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &ep, sizeof ep));
+        int32_t bt = (int32_t) type;
+        LT_TRY(hipblasLtMatmulDescSetAttribute(plan->desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bt, sizeof bt));
+        // the heuristic wants a bias pointer to be present; the real one is set per call
+        const void *dummy = ctx->workspace;
+        LT_TRY(hipblasLtMatmulDescSetAttribute(plan->desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &dummy, sizeof dummy));
+    }
+    int rc;
+    if ((rc = make_layout(&plan->a, type, k.transA ? k.K : k.M, k.transA ? k.M : k.K, k.lda, k.batch, k.strideA))) return rc;
+    if ((rc = make_layout(&plan->b, type, k.transB ? k.N : k.K, k.transB ? k.K : k.N, k.ldb, k.batch, k.strideB))) return rc;
+    if ((rc = make_layout(&plan->c, type, k.M, k.N, k.ldc, k.batch, k.strideC))) return rc;
+
+    hipblasLtMatmulPreference_t pref;
+    LT_TRY(hipblasLtMatmulPreferenceCreate(&pref));
+    uint64_t ws = kWorkspaceBytes;
+    LT_TRY(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof ws));
+    hipblasLtMatmulHeuristicResult_t found[8];
+    int n = 0;
+    hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(ctx->lt, plan->desc, plan->a, plan->b, plan->c, plan->c, pref,
+                                                         8, found, &n);
+    hipblasLtMatmulPreferenceDestroy(pref);
+    if (st != HIPBLAS_STATUS_SUCCESS || n == 0) {
+        if (getenv("CUBERT_VERBOSE")) {
+            fprintf(stderr,
+                    "hipBLASLt: no algorithm for gemm type=%d trans=%d%d M=%d N=%d K=%d lda=%d ldb=%d ldc=%d batch=%d "
+                    "bias=%d (status %d); using the plain kernel\n",
+                    k.type, k.transA, k.transB, k.M, k.N, k.K, k.lda, k.ldb, k.ldc, k.batch, (int) k.bias, (int) st);
+        }
+        plan->ok = false;
+        return 0;
+    }
+    plan->algo = found[0].algo;
+    plan->workspace = found[0].workspaceSize;
+    plan->ok = true;
+    return 0;
+}
+
+// Plain one-thread-per-output GEMM (fp32 accumulation, k ascending).  Used for shapes hipBLASLt has no
+// algorithm for (tiny or oddly aligned operands) and, with CUBERT_GEMM=naive in the environment, for all
+// of them, which gives an independent check of the hipBLASLt call convention.
+template <typename T>
+__global__ void naive_gemm_kernel(int transA, int transB, int M, int N, int K, float alpha, const T *__restrict__ A,
+                                  int lda, long long strideA, const T *__restrict__ B, int ldb, long long strideB,
+                                  float beta, T *__restrict__ C, int ldc, long long strideC, int batch,
+                                  const T *__restrict__ bias) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    const int j = blockIdx.y * blockDim.y + threadIdx.y;
+    if (i >= M || j >= N) return;
+    for (int z = blockIdx.z; z < batch; z += gridDim.z) {
+        const T *a = A + z * strideA;
+        const T *b = B + z * strideB;
+        T *c = C + z * strideC;
+        float acc = 0.f;
+        for (int k = 0; k < K; ++k) {
+            const float av = (float) (transA ? a[k + (size_t) i * lda] : a[i + (size_t) k * lda]);
+            const float bv = (float) (transB ? b[j + (size_t) k * ldb] : b[k + (size_t) j * ldb]);
+            acc += av * bv;
+        }
+        float v = alpha * acc;
+        if (beta != 0.f) v += beta * (float) c[i + (size_t) j * ldc];
+        if (bias != nullptr) v += (float) bias[i];
+        c[i + (size_t) j * ldc] = (T) v;
+    }
+}
+
+int run_naive_gemm(hipStream_t stream, int type, int transA, int transB, int M, int N, int K, float alpha,
+                   const void *A, int lda, long long strideA, const void *B, int ldb, long long strideB, float beta,
+                   void *C, int ldc, long long strideC, int batch, const void *bias) {
+    dim3 block(16, 16), grid((M + 15) / 16, (N + 15) / 16, batch < 65535 ? batch : 65535);
+    if (grid.y > 65535) return CUBERT_BAD_ARGUMENT;
+    if (type == 0) {
+        hipLaunchKernelGGL(naive_gemm_kernel<float>, grid, block, 0, stream, transA, transB, M, N, K, alpha,
+                           (const float *) A, lda, strideA, (const float *) B, ldb, strideB, beta, (float *) C, ldc,
+                           strideC, batch, (const float *) bias);
+    } else {
+        hipLaunchKernelGGL(naive_gemm_kernel<_Float16>, grid, block, 0, stream, transA, transB, M, N, K, alpha,
+                           (const _Float16 *) A, lda, strideA, (const _Float16 *) B, ldb, strideB, beta,
+                           (_Float16 *) C, ldc, strideC, batch, (const _Float16 *) bias);
+    }
+    return hip_rc(hipGetLastError());
+}
+
+bool force_naive_gemm() {
+    static const bool forced = [] {
+        const char *v = getenv("CUBERT_GEMM");
+        return v != nullptr && std::string(v) == "naive";
+    }();
+    return forced;
+}
+
+int run_gemm(void *handle, int type, int transA, int transB, int M, int N, int K, float alpha, const void *A, int lda,
+             long long strideA, const void *B, int ldb, long long strideB, float beta, void *C, int ldc,
+             long long strideC, int batch, const void *bias) {
+    BlasContext *ctx = (BlasContext *) handle;
+    if (!ctx || !A || !B || !C || M < 0 || N < 0 || K < 0 || batch < 0) return CUBERT_BAD_ARGUMENT;
+    if (M == 0 || N == 0 || batch == 0) return 0;
+    GemmKey key{type, transA, transB, M, N, K, lda, ldb, ldc, batch, strideA, strideB, strideC, bias != nullptr,
+                beta == 0.f};
+    if (force_naive_gemm()) {
+        return run_naive_gemm(ctx->stream, type, transA, transB, M, N, K, alpha, A, lda, strideA, B, ldb, strideB,
+                              beta, C, ldc, strideC, batch, bias);
+    }
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    auto it = ctx->plans.find(key);
+    if (it == ctx->plans.end()) {
+        GemmPlan plan;
+        int rc = build_plan(ctx, key, &plan);
+        if (rc) return rc;
+        it = ctx->plans.emplace(key, plan).first;
+    }
+    GemmPlan &p = it->second;
+    if (!p.ok) {
+        return run_naive_gemm(ctx->stream, type, transA, transB, M, N, K, alpha, A, lda, strideA, B, ldb, strideB,
+                              beta, C, ldc, strideC, batch, bias);
+    }
+    if (bias) {
+        LT_TRY(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof bias));
+    }
+    LT_TRY(hipblasLtMatmul(ctx->lt, p.desc, &alpha, A, p.a, B, p.b, &beta, C, p.c, C, p.c, &p.algo, ctx->workspace,
+                           kWorkspaceBytes, ctx->stream));
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int cubert_get_gpu_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void) hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
+int cubert_set_gpu(int device) { return hip_rc(hipSetDevice(device)); }
+
+int cubert_gpu_info(int device) {
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) return (int) e;
+    fprintf(stderr, "Found device %d: %s (%s), %d compute units, %.1f GiB, memory clock %d kHz, pci bus %d\n", device,
+            prop.name, prop.gcnArchName, prop.multiProcessorCount, prop.totalGlobalMem / 1073741824.0,
+            prop.memoryClockRate, prop.pciBusID);
+    return 0;
+}
+
+void *cubert_malloc(size_t size) {
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, size ? size : 1);
+    if (e != hipSuccess) {
+        size_t free_b = 0, total_b = 0;
+        (void) hipMemGetInfo(&free_b, &total_b);
+        fprintf(stderr, "HIP %s. Tried to allocate %zu (%zu total; %zu free)\n", hipGetErrorString(e), size, total_b,
+                free_b);
+        return nullptr;
+    }
+    return p;
+}
+
+int cubert_free(void *ptr) { return ptr ? hip_rc(hipFree(ptr)) : 0; }
+
+int cubert_memcpy(void *dst, const void *src, size_t n, int kind) {
+    if (n == 0) return 0;
+    return hip_rc(hipMemcpy(dst, src, n, copy_kind(kind)));
+}
+
+int cubert_memcpy_async(void *dst, const void *src, size_t n, int kind, void *stream) {
+    if (n == 0) return 0;
+    return hip_rc(hipMemcpyAsync(dst, src, n, copy_kind(kind), (hipStream_t) stream));
+}
+
+void *cubert_stream_create(void) {
+    hipStream_t s = nullptr;
+    if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) return nullptr;
+    return s;
+}
+
+int cubert_stream_destroy(void *stream) { return stream ? hip_rc(hipStreamDestroy((hipStream_t) stream)) : 0; }
+
+int cubert_stream_synchronize(void *stream) { return hip_rc(hipStreamSynchronize((hipStream_t) stream)); }
+
+void *cubert_event_create(void) {
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    return e;
+}
+
+int cubert_event_destroy(void *event) { return event ? hip_rc(hipEventDestroy((hipEvent_t) event)) : 0; }
+
+int cubert_event_record(void *event, void *stream) { return hip_rc(hipEventRecord((hipEvent_t) event, (hipStream_t) stream)); }
+
+int cubert_event_elapsed_ms(void *start, void *stop, float *ms) {
+    return hip_rc(hipEventElapsedTime(ms, (hipEvent_t) start, (hipEvent_t) stop));
+}
+
+void *cubert_blas_create(void) {
+    BlasContext *ctx = new BlasContext();
+    if (hipblasLtCreate(&ctx->lt) != HIPBLAS_STATUS_SUCCESS) {
+        delete ctx;
+        return nullptr;
+    }
+    if (hipMalloc(&ctx->workspace, kWorkspaceBytes) != hipSuccess) {
+        hipblasLtDestroy(ctx->lt);
+        delete ctx;
+        return nullptr;
+    }
+    return ctx;
+}
+
+int cubert_blas_destroy(void *handle) {
+    BlasContext *ctx = (BlasContext *) handle;
+    if (!ctx) return 0;
+    for (auto &kv : ctx->plans) {
+        GemmPlan &p = kv.second;
+        if (p.a) hipblasLtMatrixLayoutDestroy(p.a);
+        if (p.b) hipblasLtMatrixLayoutDestroy(p.b);
+        if (p.c) hipblasLtMatrixLayoutDestroy(p.c);
+        if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+    }
+    (void) hipFree(ctx->workspace);
+    hipblasLtDestroy(ctx->lt);
+    delete ctx;
+    return 0;
+}
+
+int cubert_blas_set_stream(void *handle, void *stream) {
+    if (!handle) return CUBERT_BAD_ARGUMENT;
+    ((BlasContext *) handle)->stream = (hipStream_t) stream;
+    return 0;
+}
+
+void *cubert_blas_get_stream(void *handle) { return handle ? (void *) ((BlasContext *) handle)->stream : nullptr; }
+
+int cubert_gemm_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
+                    const float *B, int ldb, float beta, float *C, int ldc, const float *bias) {
+    return run_gemm(handle, 0, transA, transB, M, N, K, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc, 0, 1, bias);
+}
+
+int cubert_gemm_f16(void *handle, int transA, int transB, int M, int N, int K, float alpha, const cubert_half *A,
+                    int lda, const cubert_half *B, int ldb, float beta, cubert_half *C, int ldc,
+                    const cubert_half *bias) {
+    return run_gemm(handle, 1, transA, transB, M, N, K, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc, 0, 1, bias);
+}
+
+int cubert_gemm_strided_batch_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha,
+                                  const float *A, int lda, long long strideA, const float *B, int ldb,
+                                  long long strideB, float beta, float *C, int ldc, long long strideC,
+                                  int batch_count) {
+    return run_gemm(handle, 0, transA, transB, M, N, K, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC,
+                    batch_count, nullptr);
+}
+
+int cubert_gemm_strided_batch_f16(void *handle, int transA, int transB, int M, int N, int K, float alpha,
+                                  const cubert_half *A, int lda, long long strideA, const cubert_half *B, int ldb,
+                                  long long strideB, float beta, cubert_half *C, int ldc, long long strideC,
+                                  int batch_count) {
+    return run_gemm(handle, 1, transA, transB, M, N, K, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC,
+                    batch_count, nullptr);
+}
+
+}  // extern "C"

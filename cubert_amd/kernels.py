@@ -1,0 +1,121 @@
+"""The fused layer kernels on torch tensors (torch is only the device allocator
+and stream here): thin wrappers over the C ABI of include/cubert_kernels.h.
+Tensors must be contiguous CUDA tensors of dtype float32 or float16; kernels run
+on torch's current stream."""
+import torch
+
+from ._lib import lib
+
+
+def _suffix(t):
+    if t.dtype == torch.float32:
+        return "f32"
+    if t.dtype == torch.float16:
+        return "f16"
+    raise TypeError("float32 or float16 expected, got %s" % t.dtype)
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    if not t.is_cuda or not t.is_contiguous():
+        raise ValueError("contiguous CUDA tensor expected")
+    return t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise RuntimeError("%s failed with code %d" % (what, rc))
+
+
+def _call(name, ref, *args):
+    fn = getattr(lib(), "%s_%s" % (name, _suffix(ref)))
+    _check(fn(*args), fn.__name__)
+
+
+def gather(ids, table):
+    """out[i] = table[ids[i]]; ids int32 or int8."""
+    out = torch.empty((ids.numel(), table.shape[1]), dtype=table.dtype, device=table.device)
+    name = "cubert_gather_i8" if ids.dtype == torch.int8 else "cubert_gather"
+    _call(name, table, _ptr(ids), ids.numel(), _ptr(table), table.shape[1], _ptr(out), _stream())
+    return out
+
+
+def embed_ln(ids, segments, word, pos, type_, beta, gamma):
+    batch, seq = ids.shape
+    hidden = word.shape[1]
+    out = torch.empty((batch, seq, hidden), dtype=word.dtype, device=word.device)
+    _call("cubert_embed_ln", word, _ptr(ids), _ptr(segments), _ptr(word), _ptr(pos), _ptr(type_), _ptr(beta),
+          _ptr(gamma), _ptr(out), batch, seq, hidden, _stream())
+    return out
+
+
+def bias_res_ln_(inout, residual, bias, beta, gamma):
+    rows, hidden = inout.numel() // inout.shape[-1], inout.shape[-1]
+    _call("cubert_bias_res_ln", inout, _ptr(inout), _ptr(residual), _ptr(bias), _ptr(beta), _ptr(gamma), rows, hidden,
+          _stream())
+    return inout
+
+
+def bias_gelu_(inout, bias):
+    rows, width = inout.numel() // inout.shape[-1], inout.shape[-1]
+    _call("cubert_bias_gelu", inout, _ptr(inout), _ptr(bias), rows, width, _stream())
+    return inout
+
+
+def mask_scale_softmax_(scores, mask, scale=1.0):
+    batch, heads, seq, seq2 = scores.shape
+    assert seq == seq2
+    _call("cubert_mask_scale_softmax", scores, _ptr(scores), _ptr(mask), float(scale), batch, heads, seq, _stream())
+    return scores
+
+
+def row_softmax(x, out=None):
+    out = torch.empty_like(x) if out is None else out
+    _call("cubert_row_softmax", x, _ptr(x), _ptr(out), x.shape[0], x.shape[1], _stream())
+    return out
+
+
+def bias_tanh_(inout, bias):
+    _call("cubert_bias_tanh", inout, _ptr(inout), _ptr(bias), inout.shape[0], inout.shape[1], _stream())
+    return inout
+
+
+def mean_pool(x):
+    batch, seq, hidden = x.shape
+    out = torch.empty((batch, hidden), dtype=x.dtype, device=x.device)
+    _call("cubert_mean_pool", x, _ptr(x), _ptr(out), batch, seq, hidden, _stream())
+    return out
+
+
+class Blas(object):
+    """A BLAS context of the runtime bound to torch's current stream."""
+
+    def __init__(self):
+        self.handle = lib().cubert_blas_create()
+        if not self.handle:
+            raise RuntimeError("cubert_blas_create failed")
+        _check(lib().cubert_blas_set_stream(self.handle, _stream()), "cubert_blas_set_stream")
+
+    def close(self):
+        if self.handle:
+            lib().cubert_blas_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        self.close()
+
+    def gemm(self, transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, bias=None):
+        """Column-major C = alpha op(A) op(B) + beta C (+ bias per row of C) on flat tensors."""
+        _call("cubert_gemm", C, self.handle, int(transA), int(transB), M, N, K, float(alpha), _ptr(A), lda, _ptr(B),
+              ldb, float(beta), _ptr(C), ldc, _ptr(bias))
+        return C
+
+    def gemm_strided_batch(self, transA, transB, M, N, K, alpha, A, lda, sA, B, ldb, sB, beta, C, ldc, sC, batch):
+        _call("cubert_gemm_strided_batch", C, self.handle, int(transA), int(transB), M, N, K, float(alpha), _ptr(A),
+              lda, sA, _ptr(B), ldb, sB, float(beta), _ptr(C), ldc, sC, batch)
+        return C

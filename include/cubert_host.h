@@ -1,0 +1,93 @@
+/*
+ * C entry points onto the host classes, for callers that cannot take a C++
+ * exception or a C++ object across their FFI (ctypes, JNA, cgo).
+ *
+ * Two groups:
+ *  1. cubert_try_*: the public API of cuBERT.h with the same arguments, but an
+ *     argument error (std::invalid_argument, std::out_of_range ...) is caught
+ *     and returned as a code; cubert_last_error() gives its message.  The
+ *     reference lets such exceptions cross the C boundary and its Cython
+ *     binding turns them into Python exceptions (python/_cuBERT.pxd:8-66,
+ *     "except +"); a ctypes/JNA caller would abort instead.
+ *  2. cubert_bert_* / cubert_transformer_*: the constructors and methods of
+ *     cuBERT::Bert<T> (reference src/cuBERT/Bert.h:17-44) and
+ *     cuBERT::Transformer<T> (reference src/cuBERT/op_att/Transformer.h:17-39)
+ *     taking the weights as parallel arrays of names and host pointers, which
+ *     is the reference's std::unordered_map<std::string, T*> spelled in C.
+ *     dtype: 0 = float weights/outputs, 1 = binary16 weights/outputs.
+ *
+ * Return codes: 0 ok, CUBERT_E_INVALID_ARGUMENT (std::invalid_argument),
+ * CUBERT_E_OUT_OF_RANGE (std::out_of_range, e.g. a missing weight name),
+ * CUBERT_E_OTHER (any other exception).
+ */
+#ifndef CUBERT_HOST_API_H
+#define CUBERT_HOST_API_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "cuBERT.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CUBERT_E_INVALID_ARGUMENT 1
+#define CUBERT_E_OUT_OF_RANGE 2
+#define CUBERT_E_OTHER 3
+
+/* Message of the last error on the calling thread ("" if none). */
+const char *cubert_last_error(void);
+
+/* ---- 1. exception-free variants of cuBERT.h -------------------------------- */
+
+/* replaces: cuBERT_open, reference src/cuBERT.cpp:23-44 */
+int cubert_try_open(const char *model_file, int max_batch_size, int seq_length, int num_hidden_layers,
+                    int num_attention_heads, int compute_type, void **model);
+/* replaces: cuBERT_compute, reference src/cuBERT.cpp:46-67 */
+int cubert_try_compute(void *model, int batch_size, int *input_ids, int8_t *input_mask, int8_t *segment_ids,
+                       void *output, int output_type, int compute_type);
+/* replaces: cuBERT_compute_m, reference src/cuBERT.cpp:69-90 */
+int cubert_try_compute_m(void *model, int batch_size, int *input_ids, int8_t *input_mask, int8_t *segment_ids,
+                         cuBERT_Output *output, int compute_type, int output_to_float);
+/* replaces: cuBERT_close, reference src/cuBERT.cpp:92-102 */
+int cubert_try_close(void *model, int compute_type);
+/* Shape facts of an opened model (hidden size, labels, seq_length) for sizing output arrays. */
+int cubert_model_info(void *model, int compute_type, int *hidden_size, int *num_labels, int *seq_length);
+
+/* ---- 2. host classes ------------------------------------------------------- */
+
+/* replaces: Bert<T>::Bert(var, ...), reference src/cuBERT/Bert.cpp:8-65 */
+int cubert_bert_create(int dtype, int n_vars, const char *const *names, const void *const *data, int max_batch_size,
+                       int seq_length, int vocab_size, int type_vocab_size, int hidden_size, int num_hidden_layers,
+                       int num_attention_heads, int intermediate_size, int num_labels, void **bert);
+/* replaces: Bert<T>::compute, reference src/cuBERT/Bert.cpp:98-136 (asynchronous) */
+int cubert_bert_compute(void *bert, int dtype, int batch_size, int *input_ids, int8_t *input_mask,
+                        int8_t *segment_ids);
+/* replaces: Bert<T>::output / output_to_float, reference src/cuBERT/Bert.cpp:185-259 (synchronises) */
+int cubert_bert_output(void *bert, int dtype, int batch_size, cuBERT_Output *output, int output_to_float);
+/* The forward pass again on the inputs the last cubert_bert_compute left on the device (no host copies;
+ * asynchronous).  No counterpart in the reference: it is the device-resident step throughput is quoted on. */
+int cubert_bert_compute_resident(void *bert, int dtype, int batch_size);
+/* Per-kernel timing with stream events: bit k of `kinds` switches kind k on (0 embed+LN, 1 bias+residual+LN,
+ * 2 bias+GELU, 3 mask+scale+softmax, 4 bias+tanh, 5 mean pool, 6 row softmax, 7 dense GEMM, 8 attention GEMM).
+ * cubert_bert_profile_read synchronises, adds the elapsed milliseconds and launch counts seen since the last
+ * read to total_ms[kind] / count[kind] (arrays of n_kinds >= 9 entries) and forgets them. */
+int cubert_bert_profile(void *bert, int dtype, unsigned kinds);
+int cubert_bert_profile_read(void *bert, int dtype, double *total_ms, int *count, int n_kinds);
+/* The HIP stream the model's work is enqueued on. */
+void *cubert_bert_stream(void *bert, int dtype);
+int cubert_bert_destroy(void *bert, int dtype);
+
+/* replaces: Transformer<T>::Transformer + compute, reference src/cuBERT/op_att/Transformer.cpp:8-132,145-175.
+ * `input` [batch, seq, hidden] and `mask` [batch, seq] are host arrays, `output` a host array of the
+ * input's size; the call copies in, runs the encoder stack, copies out and synchronises. */
+int cubert_transformer_run(int dtype, const char *var_prefix, int n_vars, const char *const *names,
+                           const void *const *data, int batch_size, int seq_length, int hidden_size,
+                           int num_hidden_layers, int num_attention_heads, int intermediate_size, const void *input,
+                           const int8_t *mask, void *output);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUBERT_HOST_API_H */

@@ -1,0 +1,164 @@
+/*
+ * Device layer of the library: the fused, bandwidth-bound layer kernels of the
+ * BERT forward pass for gfx950 (MI355X) and the small runtime they sit on.
+ * Plain C ABI: device pointers, sizes, a stream.  This is the boundary the
+ * reference draws between its host classes (.cpp) and its device code (.cu):
+ * free launchers that take raw device pointers plus `void* stream`, run
+ * asynchronously on that stream and report nothing back.
+ *
+ * Every kernel exists for fp32 storage (`_f32`) and for IEEE binary16 storage
+ * (`_f16`, arithmetic in fp32, one rounding at the store).  `cubert_half` is
+ * the 16-bit pattern of a binary16 value.
+ *
+ * Return value of every function that returns int: 0 on success; a positive
+ * hipError_t when the launch failed; CUBERT_BAD_ARGUMENT (-1) when an argument
+ * is outside what the kernel supports (nothing is launched then).  The host
+ * classes above treat any non-zero value as fatal, as the reference does with
+ * CUDA_CHECK (src/cuBERT/common.cpp:79-93).
+ *
+ * Pointers must be aligned to their element type; the fast paths additionally
+ * need 16-byte aligned rows and are selected at launch time, other shapes take
+ * a generic path with identical results.
+ */
+#ifndef CUBERT_KERNELS_H
+#define CUBERT_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t cubert_half;
+#define CUBERT_BAD_ARGUMENT (-1)
+
+/* ------------------------------------------------------------------ kernels */
+
+/* out[i, :] = table[ids[i], :]  (no bounds check on ids, as in the reference).
+ * replaces: embedding<int,T> / embedding<int8_t,T>, reference src/cuBERT/op/Embedding.h:9-15
+ * (kernel op/Embedding.cu:8-41). */
+int cubert_gather_f32(const int32_t *ids, int n, const float *table, int width, float *out, void *stream);
+int cubert_gather_f16(const int32_t *ids, int n, const cubert_half *table, int width, cubert_half *out, void *stream);
+int cubert_gather_i8_f32(const int8_t *ids, int n, const float *table, int width, float *out, void *stream);
+int cubert_gather_i8_f16(const int8_t *ids, int n, const cubert_half *table, int width, cubert_half *out, void *stream);
+
+/* BertEmbeddings in one pass:
+ *   x = word[ids[m]] + pos[m mod seq_length] + type[segments[m]]        (m < batch*seq_length)
+ *   out[m] = beta + gamma * (x - mean) / sqrt(E[x^2] - mean^2 + 1e-12)
+ * replaces: the two embedding<> launches, the k=1 position GEMM and layer_norm_ of
+ * reference src/cuBERT/op_bert/BertEmbeddings.cpp:50-66. */
+int cubert_embed_ln_f32(const int32_t *ids, const int8_t *segments, const float *word, const float *pos,
+                        const float *type, const float *beta, const float *gamma, float *out, int batch,
+                        int seq_length, int hidden, void *stream);
+int cubert_embed_ln_f16(const int32_t *ids, const int8_t *segments, const cubert_half *word,
+                        const cubert_half *pos, const cubert_half *type, const cubert_half *beta,
+                        const cubert_half *gamma, cubert_half *out, int batch, int seq_length, int hidden,
+                        void *stream);
+
+/* bias + residual + LayerNorm, in place on `inout`:
+ *   x = inout[r] + bias + residual[r];  inout[r] = beta + gamma * (x - mean) / sqrt(var + 1e-12)
+ * `bias` may be NULL (then this is exactly the reference launcher).
+ * replaces: layer_norm_<T>(in=residual, inout, rows, hidden, mean, var, beta, gamma, stream),
+ * reference src/cuBERT/op/LayerNorm.h:5-14 (kernels op/LayerNorm.cu:11-100), plus the bias
+ * prefill of Dense::_pre_compute (op/Dense.cpp:41-44). */
+int cubert_bias_res_ln_f32(float *inout, const float *residual, const float *bias, const float *beta,
+                           const float *gamma, int rows, int hidden, void *stream);
+int cubert_bias_res_ln_f16(cubert_half *inout, const cubert_half *residual, const cubert_half *bias,
+                           const cubert_half *beta, const cubert_half *gamma, int rows, int hidden,
+                           void *stream);
+
+/* bias + GELU (erf form), in place:  x = inout[r,c] + bias[c];  inout = x * 0.5 * (1 + erf(x / sqrt 2)).
+ * `bias` may be NULL.
+ * replaces: gelu<T>(N, inout, stream), reference src/cuBERT/op/GELU.h:6-7 (op/GELU.cu:14-26),
+ * plus the bias prefill of the intermediate Dense. */
+int cubert_bias_gelu_f32(float *inout, const float *bias, int rows, int width, void *stream);
+int cubert_bias_gelu_f16(cubert_half *inout, const cubert_half *bias, int rows, int width, void *stream);
+
+/* Attention mask + scale + softmax over the last axis of scores[batch, heads, seq_length, seq_length],
+ * in place:   s = scores * scale + (mask[b, k] == 0 ? -10000 : 0);   p = exp(s - max_k s) / sum_k
+ * `mask` is the caller's int8 [batch, seq_length] input mask (any non-zero byte keeps the key) and
+ * may be NULL (no masking).
+ * replaces: _not<T> + the k=1 broadcast GEMM of AttentionMask (reference src/cuBERT/op_att/
+ * AttentionMask.h:8-12, AttentionMask.cpp:41-54), the per-layer mask copy and the alpha/beta of the
+ * QK GEMM (op_att/AttentionSelf.cpp:58-60,99-101) and softmax_<T> (op/Softmax.h:8-14, five kernels
+ * in op/Softmax.cu:104-115). */
+int cubert_mask_scale_softmax_f32(float *scores, const int8_t *mask, float scale, int batch, int heads,
+                                  int seq_length, void *stream);
+int cubert_mask_scale_softmax_f16(cubert_half *scores, const int8_t *mask, float scale, int batch, int heads,
+                                  int seq_length, void *stream);
+
+/* Row softmax of a [rows, channel] matrix, in place or not (classifier probabilities).
+ * replaces: softmax_<T>(in, out, rows, channel, sum_buf, stream), reference src/cuBERT/op/Softmax.h:8-14. */
+int cubert_row_softmax_f32(const float *in, float *out, int rows, int channel, void *stream);
+int cubert_row_softmax_f16(const cubert_half *in, cubert_half *out, int rows, int channel, void *stream);
+
+/* bias + tanh, in place on [rows, width]; `bias` may be NULL.
+ * replaces: tanh_<T>(inout, N, stream), reference src/cuBERT/op_bert/BertPooler.h:8-11
+ * (op_bert/BertPooler.cu:14-26), plus the pooler's bias prefill (BertPooler.cpp:65). */
+int cubert_bias_tanh_f32(float *inout, const float *bias, int rows, int width, void *stream);
+int cubert_bias_tanh_f16(cubert_half *inout, const cubert_half *bias, int rows, int width, void *stream);
+
+/* out[b, c] = (sum_s in[b, s, c]) / seq_length  -- every position counts, padding included.
+ * replaces: reduce_mean_1<T>(in, out, batch, seq_length, hidden, stream),
+ * reference src/cuBERT/op_bert/BertPooler.h:13-16 (op_bert/BertPooler.cu:35-66). */
+int cubert_mean_pool_f32(const float *in, float *out, int batch, int seq_length, int hidden, void *stream);
+int cubert_mean_pool_f16(const cubert_half *in, cubert_half *out, int batch, int seq_length, int hidden,
+                         void *stream);
+
+/* ------------------------------------------------------------------ runtime
+ * replaces: reference src/cuBERT/common.h:17-92 (cudart + cuBLAS side). */
+
+int cubert_get_gpu_count(void);
+int cubert_set_gpu(int device);
+int cubert_gpu_info(int device); /* prints name, memory and clock to stderr */
+
+void *cubert_malloc(size_t size); /* device memory; NULL on failure */
+int cubert_free(void *ptr);
+/* kind: 1 host->device, 2 device->host, 3 device->device (cudaMemcpyKind numbering, common.h:31-40) */
+int cubert_memcpy(void *dst, const void *src, size_t n, int kind);
+int cubert_memcpy_async(void *dst, const void *src, size_t n, int kind, void *stream);
+
+void *cubert_stream_create(void);
+int cubert_stream_destroy(void *stream);
+int cubert_stream_synchronize(void *stream);
+
+/* Timing events on a stream (no counterpart in the reference, which has no built-in profiling):
+ * used to measure single kernels of a forward pass where they run. */
+void *cubert_event_create(void);
+int cubert_event_destroy(void *event);
+int cubert_event_record(void *event, void *stream);
+int cubert_event_elapsed_ms(void *start, void *stop, float *ms); /* both events must have completed */
+
+/* A BLAS context: a hipBLASLt handle, a workspace, a plan cache, bound to one stream. */
+void *cubert_blas_create(void);
+int cubert_blas_destroy(void *handle);
+int cubert_blas_set_stream(void *handle, void *stream);
+void *cubert_blas_get_stream(void *handle);
+
+/* Column-major GEMM with the meaning of cublasGemmEx / cblas_sgemm:
+ *   C = alpha * op(A) * op(B) + beta * C        (fp32 accumulation for both storage types)
+ * When `bias` is not NULL it is a length-M vector added to every column of the product before
+ * beta*C (GEMM epilogue), which is how a Dense bias is applied for row-major activations.
+ * replaces: blas_gemm<T>, reference src/cuBERT/common.h:59-68 (common.cpp:224-258,351-372). */
+int cubert_gemm_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha, const float *A,
+                    int lda, const float *B, int ldb, float beta, float *C, int ldc, const float *bias);
+int cubert_gemm_f16(void *handle, int transA, int transB, int M, int N, int K, float alpha,
+                    const cubert_half *A, int lda, const cubert_half *B, int ldb, float beta, cubert_half *C,
+                    int ldc, const cubert_half *bias);
+
+/* The same over `batch_count` problems at fixed strides (in elements).
+ * replaces: blas_gemm_strided_batch<T>, reference src/cuBERT/common.h:82-92. */
+int cubert_gemm_strided_batch_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha,
+                                  const float *A, int lda, long long strideA, const float *B, int ldb,
+                                  long long strideB, float beta, float *C, int ldc, long long strideC,
+                                  int batch_count);
+int cubert_gemm_strided_batch_f16(void *handle, int transA, int transB, int M, int N, int K, float alpha,
+                                  const cubert_half *A, int lda, long long strideA, const cubert_half *B,
+                                  int ldb, long long strideB, float beta, cubert_half *C, int ldc,
+                                  long long strideC, int batch_count);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUBERT_KERNELS_H */

@@ -1,0 +1,128 @@
+"""CPU-side checks: the shared library loads and exports exactly what include/*.h declares, the
+GraphDef writer produces files its reader (and the wire format) agree on, and the synthetic
+weight/input generators are deterministic.  No device call is made here."""
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+INCLUDE = os.path.join(ROOT, "include")
+
+
+def declared_functions():
+    names = set()
+    for header in ("cuBERT.h", "cubert_kernels.h", "cubert_host.h"):
+        text = open(os.path.join(INCLUDE, header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        text = re.sub(r"//[^\n]*", "", text)
+        names.update(re.findall(r"\b(cuBERT_\w+|cubert_\w+)\s*\(", text))
+    return names
+
+
+def test_library_exports_every_declared_symbol():
+    from cubert_amd._lib import LIB_PATH, SIGNATURES, lib
+    assert os.path.exists(LIB_PATH), "build the library first: python -m cubert_amd.build"
+    declared = declared_functions()
+    assert len(declared) > 50
+    exported = set(l.split()[-1] for l in subprocess.check_output(["nm", "-D", "--defined-only", LIB_PATH],
+                                                                   text=True).splitlines())
+    assert declared <= exported, sorted(declared - exported)
+    assert declared == set(SIGNATURES), sorted(declared ^ set(SIGNATURES))
+    lib()  # resolves every symbol through ctypes
+
+
+def test_public_header_is_valid_c_and_abi_constants():
+    """cuBERT.h must stay usable from C callers and keep the reference's enum values / field order."""
+    src = '#include "cuBERT.h"\n#include "cubert_kernels.h"\n#include "cubert_host.h"\n' \
+          '#include <stddef.h>\n' \
+          '_Static_assert(cuBERT_COMPUTE_FLOAT == 0 && cuBERT_COMPUTE_HALF == 1, "compute type");\n' \
+          '_Static_assert(cuBERT_LOGITS == 0 && cuBERT_POOLED_OUTPUT == 1 && cuBERT_SEQUENCE_OUTPUT == 2 && ' \
+          'cuBERT_EMBEDDING_OUTPUT == 3 && cuBERT_PROBS == 4, "output type");\n' \
+          '_Static_assert(offsetof(cuBERT_Output, logits) == 0 && offsetof(cuBERT_Output, pooled_output) == 8 && ' \
+          'offsetof(cuBERT_Output, sequence_output) == 16 && offsetof(cuBERT_Output, embedding_output) == 24 && ' \
+          'offsetof(cuBERT_Output, probs) == 32, "output struct");\nint main(void) { return 0; }\n'
+    subprocess.run(["gcc", "-std=c11", "-fsyntax-only", "-I", INCLUDE, "-x", "c", "-"], input=src, text=True, check=True)
+    from cubert_amd._lib import cuBERT_Output
+    assert [f[0] for f in cuBERT_Output._fields_] == ["logits", "pooled_output", "sequence_output", "embedding_output",
+                                                      "probs"]
+
+
+def test_no_gpu_reports_zero_devices_or_more():
+    from cubert_amd import get_gpu_count
+    assert get_gpu_count() >= 0
+
+
+def test_graphdef_round_trip(tmp_path):
+    from cubert_amd.graphdef import read_graphdef, write_graphdef
+    rng = np.random.default_rng(0)
+    w = {"bert/embeddings/word_embeddings": rng.normal(size=(300, 24)).astype(np.float32),
+         "output_weights": rng.normal(size=(3, 24)).astype(np.float16),
+         "output_bias": rng.normal(size=3).astype(np.float32),
+         "a/scalar": np.float32(2.5).reshape(())}
+    path = write_graphdef(str(tmp_path / "m.pb"), w)
+    back = read_graphdef(path)
+    assert set(back) == set(w)
+    for k in w:
+        assert back[k].dtype == w[k].dtype and back[k].shape == w[k].shape
+        assert np.array_equal(back[k], w[k])
+
+
+def test_graphdef_wire_format_matches_protobuf_library(tmp_path):
+    """Decode the written bytes with google.protobuf's own wire decoder (no TensorFlow schema needed):
+    field numbers GraphDef.node=1, NodeDef.name=1/op=2/attr=5, AttrValue.tensor=8, TensorProto.dtype=1/
+    tensor_shape=2/tensor_content=4."""
+    decoder = pytest.importorskip("google.protobuf.internal.decoder")
+    from cubert_amd.graphdef import write_graphdef
+    w = {"x": np.arange(6, dtype=np.float32).reshape(2, 3)}
+    buf = open(write_graphdef(str(tmp_path / "m.pb"), w), "rb").read()
+
+    def fields(b):
+        pos, out = 0, []
+        while pos < len(b):
+            tag, pos = decoder._DecodeVarint(b, pos)
+            num, wire = tag >> 3, tag & 7
+            if wire == 0:
+                v, pos = decoder._DecodeVarint(b, pos)
+            else:
+                assert wire == 2
+                n, pos = decoder._DecodeVarint(b, pos)
+                v, pos = b[pos:pos + n], pos + n
+            out.append((num, v))
+        return out
+
+    node = dict(fields(buf))[1]
+    nf = fields(node)
+    assert (1, b"x") in nf and (2, b"Const") in nf
+    attrs = {dict(fields(v))[1]: dict(fields(v))[2] for n, v in nf if n == 5}
+    tensor = dict(fields(dict(fields(attrs[b"value"]))[8]))
+    assert tensor[1] == 1  # DT_FLOAT
+    dims = [dict(fields(v))[1] for n, v in fields(tensor[2]) if n == 2]
+    assert dims == [2, 3]
+    assert np.array_equal(np.frombuffer(tensor[4], np.float32), np.arange(6, dtype=np.float32))
+
+
+def test_generators_are_deterministic_and_follow_the_configs():
+    from cubert_amd.testing import CONFIGS, config_inputs, random_bert_weights
+    small = dict(vocab=50, hidden=16, layers=2, heads=2, intermediate=32, max_position=8, type_vocab=2)
+    a = random_bert_weights(seed=1, **small)
+    b = random_bert_weights(seed=1, **small)
+    assert all(np.array_equal(a[k], b[k]) for k in a)
+    assert a["bert/embeddings/word_embeddings"].shape == (50, 16)
+    assert a["bert/encoder/layer_1/intermediate/dense/kernel"].shape == (16, 32)
+    assert a["output_weights"].shape == (2, 16)
+    assert abs(a["bert/embeddings/word_embeddings"].std() - 0.02) < 0.003
+    assert (a["bert/encoder/layer_0/output/LayerNorm/gamma"] == 1).all()
+    ids, mask, seg = config_inputs("C1")
+    assert ids.shape == (128, 32) and ids.dtype == np.int32 and mask.dtype == np.int8 and seg.dtype == np.int8
+    assert ids.min() >= 0 and ids.max() < 21128
+    valid = mask.sum(1)
+    assert valid.min() >= 8 and valid.max() <= 32 and (np.diff(mask.astype(int), axis=1) <= 0).all()
+    assert (seg[:, :16] == 0).all() and (seg[:, 16:] == 1).all()
+    ids3, mask3, _ = config_inputs("C3")
+    assert ids3.shape == (64, 512) and mask3.sum(1).min() >= 16
+    _, mask4, seg4 = config_inputs("C4")
+    assert mask4.all() and (seg4[:, 0] == 0).all() and (seg4[:, -1] == 1).all()
+    assert set(CONFIGS) == {"C0", "C1", "C2", "C3", "C4"}

@@ -1,0 +1,358 @@
+"""Parity of every fused kernel, called through the C ABI (include/cubert_kernels.h),
+against the CPU oracle on the same seeded inputs, plus the known-answer vectors of the
+reference's unit tests and the edge cases it covers.  fp32: 1e-5 relative (norm-wise);
+fp16 storage: compared with the oracle run on the fp16-rounded inputs, within fp16
+output rounding (2e-3 relative)."""
+import math
+
+import numpy as np
+import pytest
+
+import oracle
+from util import FP32_TOL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+T = "test/cuBERT/"
+F16_KERNEL_TOL = 2e-3
+
+
+@pytest.fixture(scope="module")
+def K():
+    if not torch.cuda.is_available():
+        pytest.fail("no GPU visible: the -m gpu tests must run on the MI355X box")
+    from cubert_amd import kernels
+    return kernels
+
+
+def dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.float().cpu().numpy()
+
+
+def tdt(name):
+    return torch.float32 if name == "f32" else torch.float16
+
+
+def q(a, name):
+    """The values the kernel actually sees: fp32, or fp32 rounded to fp16 and back."""
+    a = np.asarray(a, np.float32)
+    return a if name == "f32" else oracle.round_to_half(a)
+
+
+def tol(name):
+    return FP32_TOL if name == "f32" else F16_KERNEL_TOL
+
+
+# ------------------------------------------------------------------ reference vectors
+
+def test_layer_norm_reference_vector(K, case):
+    c = case(T + "op/LayerNormTest.cpp", "layer_norm_ext")
+    inout = dev(np.array(c.arrays["inout"], np.float32).reshape(2, 3))
+    K.bias_res_ln_(inout, dev(np.array(c.arrays["in"], np.float32).reshape(2, 3)), None,
+                   dev(np.array(c.arrays["beta"], np.float32)), dev(np.array(c.arrays["gamma"], np.float32)))
+    c.check(host(inout))
+
+
+def test_softmax_reference_vector(K, case):
+    c = case(T + "op/SoftmaxTest.cpp", "softmax_")
+    x = dev(np.array(c.arrays["inout"], np.float32).reshape(2, 3))
+    c.check(host(K.row_softmax(x)))
+    # the same rows through the attention kernel (square score matrix, no mask, scale 1)
+    s3 = torch.zeros((1, 1, 3, 3), device="cuda")
+    s3[0, 0, :2] = x
+    K.mask_scale_softmax_(s3, None, 1.0)
+    c.check(host(s3)[0, 0, :2])
+
+
+def test_gelu_reference_vector(K, case):
+    c = case(T + "op/GELUTest.cpp", "gelu")
+    x = np.array(c.arrays["inout"], np.float32)
+    y = dev(x.reshape(1, 5).copy())
+    K.bias_gelu_(y, None)
+    c.check(host(y), closed_form=lambda i: x[i] * 0.5 * (1.0 + math.erf(x[i] / math.sqrt(2.0))))
+
+
+def test_embedding_reference_vector(K, case):
+    c = case(T + "op/EmbeddingTest.cpp", "embedding")
+    out = K.gather(dev(np.array(c.arrays["input_ids"], np.int32)),
+                   dev(np.array(c.arrays["embedding_table"], np.float32).reshape(4, 3)))
+    c.check(host(out))
+
+
+def test_bert_embeddings_reference_vector(K, case):
+    c = case(T + "op_bert/BertEmbeddingsTest.cpp", "bert_embedding")
+    f = lambda k, *s: dev(np.array(c.arrays[k], np.float32).reshape(*s))
+    out = K.embed_ln(dev(np.array(c.arrays["input_ids"], np.int32).reshape(2, 4)),
+                     dev(np.array(c.arrays["segment_ids"], np.int8).reshape(2, 4)),
+                     f("word_embeddings", 5, 3), f("position_embeddings", 4, 3), f("token_type_embeddings", 2, 3),
+                     f("beta", 3), f("gamma", 3))
+    c.check(host(out))
+
+
+def test_pooler_reference_vectors(K, case):
+    c = case(T + "op_bert/BertPoolerTest.cpp", "bert_pooler")
+    x = dev(np.array(c.arrays["in"], np.float32).reshape(2, 3, 2))
+    kernel = dev(np.array(c.arrays["kernel"], np.float32).reshape(2, 2))
+    out = torch.zeros((2, 2), device="cuda")
+    blas = K.Blas()
+    # first token of each sequence: ldb = hidden * seq_length, as the reference's pooler GEMM
+    blas.gemm(False, False, 2, 2, 2, 1.0, kernel, 2, x, 2 * 3, 0.0, out, 2)
+    K.bias_tanh_(out, dev(np.array(c.arrays["bias"], np.float32)))
+    c.check(host(out))
+    c = case(T + "op_bert/BertPoolerTest.cpp", "mean_pooler")
+    c.check(host(K.mean_pool(dev(np.array(c.arrays["in"], np.float32).reshape(2, 3, 2)))))
+
+
+def test_dense_reference_vector(K, case):
+    c = case(T + "op/DenseTest.cpp", "dense")
+    kernel = dev(np.array(c.arrays["kernel"], np.float32))
+    x = dev(np.array(c.arrays["input"], np.float32))
+    out = torch.zeros(9, device="cuda")
+    K.Blas().gemm(False, False, 3, 3, 2, 1.0, kernel, 3, x, 2, 0.0, out, 3, bias=dev(np.array(c.arrays["bias"], np.float32)))
+    c.check(host(out))
+
+
+def test_attention_mask_reference_vector(K, case):
+    """AttentionMaskTest pins neg = !mask broadcast over heads and queries.  The fused kernel never
+    materialises that tensor; what it must reproduce is its effect: with all scores zero, keys with
+    neg = 1 get the -10000 addend, i.e. probability exp(-10000) = 0 unless every key of the row is masked."""
+    c = case(T + "op_att/AttentionMaskTest.cpp", "attention_mask")
+    mask = np.array(c.arrays["in"], np.int8).reshape(2, 2)
+    neg = np.array([v for _, _, v, _ in c.expect], np.float32).reshape(2, 3, 2, 2)  # [b, a, q, k]
+    scores = torch.zeros((2, 3, 2, 2), device="cuda")
+    K.mask_scale_softmax_(scores, dev(mask), 1.0)
+    want = oracle.softmax_((-10000.0 * neg).reshape(-1, 2)).reshape(2, 3, 2, 2)
+    np.testing.assert_allclose(host(scores), want, atol=1e-7)
+    assert host(scores)[0, :, :, 0].min() == 1.0 and host(scores)[0, :, :, 1].max() == 0.0
+    np.testing.assert_allclose(host(scores)[1], 0.5)  # fully masked rows stay uniform
+
+
+def test_batch_matmul_reference_vectors(K, case):
+    """QK^T and PV layouts of BatchMatMulTest through the strided-batched GEMM, both loop orders."""
+    blas = K.Blas()
+    S, A, d, B = 2, 4, 3, 2
+    H = A * d
+    c = case(T + "op_att/BatchMatMulTest.cpp", "q_k")
+    qh, kh = np.array(c.arrays["query"], np.float32), np.array(c.arrays["key"], np.float32)
+    want = oracle.att_q_k(qh, kh, B, S, A, d)  # [B, S_q, A, S_k], pinned by the oracle test
+    c.check(want)
+    q_, k_ = dev(qh), dev(kh)
+    for loop_heads in (True, False):
+        out = torch.zeros(B * A * S * S, device="cuda")  # [B, A, S_q, S_k]
+        if loop_heads:
+            for a in range(A):
+                blas.gemm_strided_batch(True, False, S, S, d, 1.0, k_[a * d:], H, S * H, q_[a * d:], H, S * H, 0.0,
+                                        out[a * S * S:], S, A * S * S, B)
+        else:
+            for b in range(B):
+                blas.gemm_strided_batch(True, False, S, S, d, 1.0, k_[b * S * H:], H, d, q_[b * S * H:], H, d, 0.0,
+                                        out[b * A * S * S:], S, S * S, A)
+        got = host(out).reshape(B, A, S, S).transpose(0, 2, 1, 3)
+        np.testing.assert_array_equal(got, want)
+    c = case(T + "op_att/BatchMatMulTest.cpp", "qk_v")
+    p_h, v_h = np.array(c.arrays["qk"], np.float32), np.array(c.arrays["value"], np.float32)
+    want = oracle.att_qk_v(p_h, v_h, B, S, A, d)
+    c.check(want)
+    p_ = dev(np.ascontiguousarray(p_h.reshape(B, S, A, S).transpose(0, 2, 1, 3)))  # ours: [B, A, S_q, S_k]
+    v_ = dev(v_h)
+    out = torch.zeros(B * S * H, device="cuda")
+    for a in range(A):
+        blas.gemm_strided_batch(False, False, d, S, S, 1.0, v_[a * d:], H, S * H, p_.reshape(-1)[a * S * S:], S,
+                                A * S * S, 0.0, out[a * d:], H, S * H, B)
+    np.testing.assert_array_equal(host(out).reshape(B, S, A, d), want)
+
+
+# ------------------------------------------------------------------ seeded parity with the oracle
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("rows,hidden", [(4096, 768), (1000, 1024), (37, 768), (5, 256), (64, 1280), (3, 6), (9, 100),
+                                         (2, 4096)])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_bias_res_ln(K, name, rows, hidden, with_bias):
+    rng = np.random.default_rng(rows * 7 + hidden)
+    x = q(rng.normal(0.2, 1.5, (rows, hidden)), name)
+    res = q(rng.normal(0, 1, (rows, hidden)), name)
+    bias = q(rng.normal(0, 0.5, hidden), name)
+    beta = q(rng.normal(0, 0.3, hidden), name)
+    gamma = q(rng.normal(1, 0.2, hidden), name)
+    inout = dev(x, tdt(name))
+    K.bias_res_ln_(inout, dev(res, tdt(name)), dev(bias, tdt(name)) if with_bias else None, dev(beta, tdt(name)),
+                   dev(gamma, tdt(name)))
+    # the reference adds the bias into the GEMM output first, then LayerNorm adds the residual
+    pre = x + bias if with_bias else x
+    want = oracle.layer_norm_(res, pre, beta, gamma)
+    assert_close(host(inout), want, tol(name), "bias_res_ln %s" % name)
+
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("batch,seq,hidden,vocab", [(128, 32, 768, 21128), (3, 128, 1024, 3000), (2, 4, 6, 11),
+                                                    (1, 512, 768, 21128), (5, 7, 100, 50)])
+def test_embed_ln(K, name, batch, seq, hidden, vocab):
+    rng = np.random.default_rng(batch + seq + hidden)
+    w = {"bert/embeddings/word_embeddings": q(rng.normal(0, 0.02, (vocab, hidden)), name),
+         "bert/embeddings/token_type_embeddings": q(rng.normal(0, 0.02, (2, hidden)), name),
+         "bert/embeddings/position_embeddings": q(rng.normal(0, 0.02, (seq, hidden)), name),
+         "bert/embeddings/LayerNorm/beta": q(rng.normal(0, 0.1, hidden), name),
+         "bert/embeddings/LayerNorm/gamma": q(rng.normal(1, 0.1, hidden), name)}
+    ids = rng.integers(0, vocab, (batch, seq), dtype=np.int32)
+    ids[0, 0], ids[-1, -1] = 0, vocab - 1
+    seg = rng.integers(0, 2, (batch, seq)).astype(np.int8)
+    d = lambda k: dev(w["bert/embeddings/" + k], tdt(name))
+    out = K.embed_ln(dev(ids), dev(seg), d("word_embeddings"), d("position_embeddings"), d("token_type_embeddings"),
+                     d("LayerNorm/beta"), d("LayerNorm/gamma"))
+    want = oracle.bert_embeddings(w, ids, seg, batch, seq, hidden).reshape(batch, seq, hidden)
+    assert_close(host(out), want, tol(name), "embed_ln %s" % name)
+
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("rows,width", [(4096, 3072), (512, 4096), (3, 3072), (7, 5), (33, 72), (1, 8)])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_bias_gelu(K, name, rows, width, with_bias):
+    rng = np.random.default_rng(rows + width)
+    x = q(rng.normal(0, 2.5, (rows, width)), name)
+    x.ravel()[:6] = q(np.array([-12, -6, -0.0, 0.0, 6, 12]), name)[: min(6, x.size)]
+    bias = q(rng.normal(0, 0.5, width), name)
+    y = dev(x, tdt(name))
+    K.bias_gelu_(y, dev(bias, tdt(name)) if with_bias else None)
+    want = oracle.gelu(x + bias if with_bias else x)
+    assert_close(host(y), want, tol(name), "bias_gelu %s" % name)
+
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("batch,heads,seq", [(128, 12, 32), (8, 12, 128), (2, 12, 512), (2, 2, 4), (3, 5, 7),
+                                             (2, 3, 384), (1, 16, 64), (2, 4, 8), (2, 2, 1024), (1, 2, 100)])
+def test_mask_scale_softmax(K, name, batch, heads, seq):
+    rng = np.random.default_rng(batch * 131 + heads * 17 + seq)
+    raw = q(rng.normal(0, 6, (batch, heads, seq, seq)), name)
+    valid = rng.integers(1, seq + 1, batch)
+    mask = (np.arange(seq)[None, :] < valid[:, None]).astype(np.int8)
+    mask[0] = (rng.random(seq) < 0.5)  # a scattered pattern, and values other than 1
+    mask[0, rng.integers(0, seq)] = 3
+    scale = 0.125
+    s = dev(raw, tdt(name))
+    K.mask_scale_softmax_(s, dev(mask), scale)
+    neg = oracle.not_(mask)  # 1.0 where the key is masked
+    logits = raw * np.float32(scale) + np.float32(-10000.0) * neg[:, None, None, :]
+    want = oracle.softmax_(logits.reshape(-1, seq)).reshape(raw.shape)
+    got = host(s)
+    assert_close(got, want, tol(name), "mask_scale_softmax %s" % name)
+    np.testing.assert_allclose(got.sum(-1), 1.0, atol=1e-5 if name == "f32" else 4e-3)
+    assert got[0][:, :, mask[0] == 0].max() == 0.0  # masked keys get exactly zero probability
+
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+def test_mask_special_cases(K, name):
+    rng = np.random.default_rng(0)
+    raw = q(rng.normal(0, 3, (2, 2, 32, 32)), name)
+    ones = np.ones((2, 32), np.int8)
+    plain = oracle.softmax_(raw.reshape(-1, 32)).reshape(raw.shape)
+    a = dev(raw, tdt(name)); K.mask_scale_softmax_(a, dev(ones), 1.0)      # all kept = plain softmax
+    b = dev(raw, tdt(name)); K.mask_scale_softmax_(b, None, 1.0)           # no mask at all
+    assert_close(host(a), plain, tol(name))
+    assert np.array_equal(host(a), host(b))
+    # every key masked: the -10000 shift cancels up to fp32 rounding at magnitude 1e4
+    z = dev(raw, tdt(name)); K.mask_scale_softmax_(z, dev(np.zeros((2, 32), np.int8)), 1.0)
+    want = oracle.softmax_((raw - np.float32(10000.0)).reshape(-1, 32)).reshape(raw.shape)
+    assert_close(host(z), want, tol(name))
+
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("rows,channel", [(128, 2), (256, 3), (1, 1), (77, 16), (40, 33), (5, 1000)])
+def test_row_softmax(K, name, rows, channel):
+    rng = np.random.default_rng(rows + channel)
+    x = q(rng.normal(0, 4, (rows, channel)), name)
+    got = host(K.row_softmax(dev(x, tdt(name))))
+    assert_close(got, oracle.softmax_(x), tol(name), "row_softmax")
+
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("rows,width", [(128, 768), (256, 1024), (1, 768), (3, 5)])
+def test_bias_tanh(K, name, rows, width):
+    rng = np.random.default_rng(rows + width)
+    x = q(rng.normal(0, 2, (rows, width)), name)
+    bias = q(rng.normal(0, 0.5, width), name)
+    y = dev(x, tdt(name))
+    K.bias_tanh_(y, dev(bias, tdt(name)))
+    assert_close(host(y), oracle.tanh_(x + bias), tol(name), "bias_tanh")
+
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("batch,seq,hidden", [(32, 128, 768), (4, 512, 1024), (2, 3, 2), (3, 5, 100), (1, 1, 768)])
+def test_mean_pool(K, name, batch, seq, hidden):
+    rng = np.random.default_rng(batch + seq + hidden)
+    x = q(rng.normal(0.1, 1, (batch, seq, hidden)), name)
+    got = host(K.mean_pool(dev(x, tdt(name))))
+    assert_close(got, oracle.reduce_mean_1(x), tol(name), "mean_pool")
+
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("idt", [np.int32, np.int8])
+def test_gather(K, name, idt):
+    rng = np.random.default_rng(1)
+    table = q(rng.normal(0, 1, (100, 768)), name)
+    ids = rng.integers(0, 100, 333).astype(idt)
+    got = host(K.gather(dev(ids), dev(table, tdt(name))))
+    assert np.array_equal(got, oracle.embedding(ids, table))  # a copy: bit exact
+
+
+# ------------------------------------------------------------------ GEMM convention
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
+@pytest.mark.parametrize("M,N,K_", [(768, 4096, 768), (2, 128, 768), (5, 7, 11), (3072, 64, 768)])
+def test_gemm_against_oracle_sgemm(K, name, ta, tb, M, N, K_):
+    rng = np.random.default_rng(M + N + K_ + ta * 2 + tb)
+    lda, ldb, ldc = (K_ if ta else M), (N if tb else K_), M
+    A = q(rng.normal(0, 1, lda * (M if ta else K_)), name)
+    B = q(rng.normal(0, 1, ldb * (K_ if tb else N)), name)
+    C0 = q(rng.normal(0, 1, ldc * N), name)
+    bias = q(rng.normal(0, 1, M), name)
+    blas = K.Blas()
+    for beta, use_bias in ((0.0, False), (1.0, False), (0.0, True)):
+        C = dev(C0, tdt(name))
+        blas.gemm(ta, tb, M, N, K_, 0.5, dev(A, tdt(name)), lda, dev(B, tdt(name)), ldb, beta, C, ldc,
+                  bias=dev(bias, tdt(name)) if use_bias else None)
+        want = oracle.sgemm(ta, tb, M, N, K_, 0.5, A, lda, B, ldb, beta, C0.copy(), ldc)
+        if use_bias:
+            want = (want.reshape(N, M) + bias[None, :]).ravel()
+        # fp32: summation order differs between BLAS libraries; error grows like sqrt(K) * eps
+        assert_close(host(C), want, 2e-5 if name == "f32" else 2e-3, "gemm %s beta=%g bias=%s" % (name, beta, use_bias))
+
+
+# ------------------------------------------------------------------ edge cases
+
+def test_empty_and_bad_arguments(K):
+    from cubert_amd._lib import lib
+    L = lib()
+    x = torch.zeros((4, 768), device="cuda")
+    assert L.cubert_bias_res_ln_f32(x.data_ptr(), x.data_ptr(), None, x.data_ptr(), x.data_ptr(), 0, 768, None) == 0
+    assert L.cubert_bias_gelu_f32(x.data_ptr(), None, 0, 768, None) == 0
+    assert L.cubert_mask_scale_softmax_f32(x.data_ptr(), None, 1.0, 0, 12, 32, None) == 0
+    assert L.cubert_bias_res_ln_f32(None, x.data_ptr(), None, x.data_ptr(), x.data_ptr(), 4, 768, None) == -1
+    assert L.cubert_bias_gelu_f32(x.data_ptr(), None, 4, 0, None) == -1
+    assert L.cubert_mask_scale_softmax_f32(x.data_ptr(), None, 1.0, 1, 0, 32, None) == -1
+    assert L.cubert_mean_pool_f32(x.data_ptr(), x.data_ptr(), 1, 0, 768, None) == -1
+    torch.cuda.synchronize()
+
+
+def test_unaligned_views_take_the_generic_path(K):
+    """Tensors offset by one element break 16-byte alignment; results must not change."""
+    rng = np.random.default_rng(5)
+    base = torch.zeros(4 * 768 + 1, device="cuda")
+    x = rng.normal(0, 1, (4, 768)).astype(np.float32)
+    base[1:] = dev(x).reshape(-1)
+    view = base[1:].view(4, 768)
+    res = dev(rng.normal(0, 1, (4, 768)).astype(np.float32))
+    beta, gamma = dev(np.zeros(768, np.float32)), dev(np.ones(768, np.float32))
+    K.bias_res_ln_(view, res, None, beta, gamma)
+    want = oracle.layer_norm_(host(res), x, np.zeros(768), np.ones(768))
+    assert_close(host(view), want, FP32_TOL)

@@ -1,0 +1,260 @@
+"""End-to-end parity of the host classes (Transformer, Bert, BertM behind cuBERT_open) with the
+CPU oracle, through the C ABI: the reference's encoder known-answer vectors, seeded random models
+at small and full BERT-base / BERT-large shapes, every output type, the GraphDef file path and the
+error behaviour of the public API.
+
+Tolerances: fp32 within 1e-5 relative (norm-wise) of the oracle; fp16 storage within 1e-2 relative
+on pooled / logit outputs of the fp32 oracle run on the same weights rounded to fp16 (the
+reference's own fp16-vs-fp32 bound, BertTest.cpp:109-110)."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from test_oracle_golden import transformer_weights
+from util import FP16_TOL, FP32_TOL, assert_close, rel_err
+
+pytestmark = pytest.mark.gpu
+
+T = "test/cuBERT/"
+
+
+@pytest.fixture(scope="module")
+def cb():
+    import torch
+    if not torch.cuda.is_available():
+        pytest.fail("no GPU visible: the -m gpu tests must run on the MI355X box")
+    import cubert_amd
+    return cubert_amd
+
+
+# ------------------------------------------------------------------ reference encoder vectors
+
+@pytest.mark.parametrize("name,layers", [("transformer", 1), ("transformer_complex", 2)])
+def test_transformer_reference_vectors(cb, case, name, layers):
+    c = case(T + "op_att/TransformerTest.cpp", name)
+    mask = np.ones((2, 4), np.int8)
+    mask[0, 0] = 0
+    out = cb.transformer_run(transformer_weights(c, layers), "encoder",
+                             np.array(c.arrays["tensor"], np.float32).reshape(2, 4, 6), mask, layers, 2, 5)
+    assert c.check(out) == 12  # the reference's own tolerances: 1e-6 (1 layer), 1e-5 (2 layers)
+
+
+def test_transformer_reference_vectors_half(cb, case):
+    c = case(T + "op_att/TransformerTest.cpp", "transformer_complex_half")
+    mask = np.ones((2, 4), np.int8)
+    mask[0, 0] = 0
+    out = cb.transformer_run(transformer_weights(c, 2), "encoder",
+                             np.array(c.arrays["tensor"], np.float32).reshape(2, 4, 6), mask, 2, 2, 5,
+                             compute_type=cb.ComputeType.HALF)
+    assert c.check(out.astype(np.float32)) == 12  # 1e-3 .. 1e-2 absolute, as the reference asserts for half
+
+
+def test_missing_weight_raises_like_unordered_map_at(cb, case):
+    c = case(T + "op_att/TransformerTest.cpp", "transformer")
+    w = transformer_weights(c, 1)
+    del w["encoder/layer_0/output/dense/bias"]
+    with pytest.raises(IndexError):
+        cb.transformer_run(w, "encoder", np.zeros((2, 4, 6), np.float32), np.ones((2, 4), np.int8), 1, 2, 5)
+
+
+# ------------------------------------------------------------------ seeded models vs the oracle
+
+SMALL = dict(vocab=211, hidden=128, layers=3, heads=4, intermediate=512, max_position=64, type_vocab=2)
+
+
+def run_both(cb, weights, ids, mask, seg, layers, heads, max_batch, compute_type=0, oracle_rows=None):
+    from cubert_amd.testing import random_bert_weights  # noqa: F401  (kept importable for -k runs)
+    S = ids.shape[1]
+    bert = cb.Bert(weights, max_batch, S, layers, heads, compute_type)
+    got = bert.forward(ids, mask, seg)
+    bert.close()
+    if compute_type == 1:
+        weights = {k: oracle.round_to_half(v) for k, v in weights.items()}
+    n = ids.shape[0] if oracle_rows is None else oracle_rows
+    want = oracle.bert_forward(weights, ids[:n], mask[:n], seg[:n], layers, heads)
+    return got, want, n
+
+
+@pytest.mark.parametrize("pooler,bias,scattered", [(True, True, False), (False, False, True), (True, False, True)])
+def test_small_model_all_outputs_fp32(cb, pooler, bias, scattered):
+    from cubert_amd.testing import random_bert_weights, random_inputs
+    w = random_bert_weights(seed=3, labels=3, pooler=pooler, classifier=True, classifier_bias=bias, ln_random=True,
+                            **SMALL)
+    ids, mask, seg = random_inputs(seed=4, batch=7, seq_length=32, vocab=SMALL["vocab"], min_valid=2,
+                                   segment_split="random", scattered_mask=scattered)
+    got, want, _ = run_both(cb, w, ids, mask, seg, 3, 4, max_batch=9)
+    for k in ("embedding_output", "sequence_output", "pooled_output", "logits", "probs"):
+        assert_close(got[k], want[k], FP32_TOL, k)
+
+
+def test_small_model_fp16(cb):
+    from cubert_amd.testing import random_bert_weights, random_inputs
+    w = random_bert_weights(seed=5, labels=2, pooler=True, classifier=True, ln_random=True, **SMALL)
+    ids, mask, seg = random_inputs(seed=6, batch=8, seq_length=64, vocab=SMALL["vocab"], min_valid=5, segment_split=20)
+    got, want, _ = run_both(cb, w, ids, mask, seg, 3, 4, max_batch=8, compute_type=1)
+    for k in ("pooled_output", "logits", "probs", "sequence_output", "embedding_output"):
+        assert_close(got[k], want[k], FP16_TOL, k)
+
+
+def test_repeated_calls_and_smaller_batches_reuse_buffers(cb):
+    """The reference's BertMTest calls one model four times; results must not depend on what ran before."""
+    from cubert_amd.testing import random_bert_weights, random_inputs
+    w = random_bert_weights(seed=7, labels=2, **SMALL)
+    ids, mask, seg = random_inputs(seed=8, batch=6, seq_length=32, vocab=SMALL["vocab"], min_valid=4)
+    bert = cb.Bert(w, 6, 32, 3, 4)
+    first = bert.forward(ids, mask, seg)
+    small = bert.forward(ids[:2], mask[:2], seg[:2])
+    again = bert.forward(ids, mask, seg)
+    bert.close()
+    for k in first:
+        assert np.array_equal(first[k], again[k]), k
+        # rows of a batch are independent of the batch they are computed in (different GEMM shapes: not bit-equal)
+        assert_close(small[k], first[k][:2], FP32_TOL, k)
+
+
+CONFIG_CASES = [
+    # name, oracle rows (None = all; rows of a batch are independent, so a prefix is enough at big shapes)
+    ("C0", None),
+    ("C1", None),
+    ("C2", 8),
+    ("C3", 2),
+    ("C4", 4),
+]
+
+
+@pytest.mark.parametrize("name,rows", CONFIG_CASES)
+def test_benchmark_configurations(cb, name, rows):
+    """The five workloads at their real shapes (BERT-base / BERT-large, random-init N(0, 0.02))."""
+    from cubert_amd.testing import CONFIGS, config_inputs, config_weights
+    cfg = CONFIGS[name]
+    m = cfg["model"]
+    w = config_weights(name, seed=0)
+    ids, mask, seg = config_inputs(name, seed=0)
+    half = cfg["dtype"] == "f16"
+    got, want, n = run_both(cb, w, ids, mask, seg, m["layers"], m["heads"], cfg["batch"], int(half), oracle_rows=rows)
+    tol = FP16_TOL if half else FP32_TOL
+    report = {}
+    for k in ("pooled_output", "logits", "probs") + (() if half else ("sequence_output", "embedding_output")):
+        report[k] = assert_close(got[k][:n], want[k], tol, "%s %s" % (name, k))
+    if half:  # token-level outputs of the fp16 path: reported, bounded loosely (no reference bound exists)
+        for k in ("sequence_output", "embedding_output"):
+            report[k] = rel_err(got[k][:n], want[k])
+            assert report[k] < 5e-2, (k, report[k])
+    print("\n%s relative errors vs oracle: %s" % (name, {k: "%.2e" % v for k, v in report.items()}))
+    # size-independent properties at the full batch
+    np.testing.assert_allclose(got["probs"].sum(-1), 1.0, atol=2e-3 if half else 1e-5)
+    assert np.isfinite(got["sequence_output"]).all()
+    if cfg["pooler"]:
+        assert np.abs(got["pooled_output"]).max() <= 1.0
+    else:
+        np.testing.assert_allclose(got["pooled_output"], got["sequence_output"].mean(1), atol=2e-3)
+    # LayerNorm with gamma = 1, beta = 0: every output row has mean 0 and variance 1
+    seq = got["sequence_output"].astype(np.float64)
+    np.testing.assert_allclose(seq.mean(-1), 0.0, atol=2e-3 if half else 1e-5)
+    np.testing.assert_allclose(seq.var(-1), 1.0, atol=1e-2 if half else 1e-4)
+
+
+# ------------------------------------------------------------------ the public C API on a GraphDef file
+
+@pytest.fixture(scope="module")
+def small_pb(tmp_path_factory):
+    from cubert_amd.graphdef import write_graphdef
+    from cubert_amd.testing import random_bert_weights
+    w = random_bert_weights(seed=9, labels=2, **SMALL)
+    path = str(tmp_path_factory.mktemp("pb") / "bert_small.pb")
+    write_graphdef(path, w)
+    return path, w
+
+
+def test_open_compute_every_output_type(cb, small_pb):
+    from cubert_amd.testing import random_inputs
+    path, w = small_pb
+    ids, mask, seg = random_inputs(seed=10, batch=5, seq_length=32, vocab=SMALL["vocab"], min_valid=3, segment_split=9)
+    want = oracle.bert_forward(w, ids, mask, seg, 3, 4)
+    model = cb.Model(path, 8, 32, 3, 4)
+    assert (model.hidden_size, model.num_labels, model.seq_length) == (128, 2, 32)
+    shapes = {cb.OutputType.LOGITS: ("logits", (5, 2)), cb.OutputType.PROBS: ("probs", (5, 2)),
+              cb.OutputType.POOLED_OUTPUT: ("pooled_output", (5, 128)),
+              cb.OutputType.SEQUENCE_OUTPUT: ("sequence_output", (5, 32, 128)),
+              cb.OutputType.EMBEDDING_OUTPUT: ("embedding_output", (5, 32, 128))}
+    for ot, (key, shape) in shapes.items():
+        out = np.zeros(shape, np.float32)
+        model.compute(ids, mask, seg, out, ot)
+        assert_close(out, want[key], FP32_TOL, key)
+    # several outputs in one call
+    o = cb.Output()
+    o.logits = np.zeros((5, 2), np.float32)
+    o.sequence_output = np.zeros((5, 32, 128), np.float32)
+    model.compute_m(ids, mask, seg, o)
+    assert_close(o.logits, want["logits"], FP32_TOL)
+    assert_close(o.sequence_output, want["sequence_output"], FP32_TOL)
+    model.close()
+
+
+def test_open_half_and_output_to_float(cb, small_pb):
+    from cubert_amd.testing import random_inputs
+    path, w = small_pb
+    ids, mask, seg = random_inputs(seed=11, batch=4, seq_length=32, vocab=SMALL["vocab"], min_valid=3)
+    want = oracle.bert_forward({k: oracle.round_to_half(v) for k, v in w.items()}, ids, mask, seg, 3, 4)
+    model = cb.Model(path, 4, 32, 3, 4, cb.ComputeType.HALF)  # float file converted to half at load
+    out16 = np.zeros((4, 2), np.float16)
+    model.compute(ids, mask, seg, out16, cb.OutputType.LOGITS)
+    o = cb.Output()
+    o.logits = np.zeros((4, 2), np.float32)
+    o.pooled_output = np.zeros((4, 128), np.float32)
+    model.compute_m(ids, mask, seg, o, output_to_float=True)
+    model.close()
+    assert_close(out16.astype(np.float32), want["logits"], FP16_TOL)
+    assert np.array_equal(out16.astype(np.float32), o.logits)
+    assert_close(o.pooled_output, want["pooled_output"], FP16_TOL)
+
+
+def test_api_error_behaviour(cb, small_pb):
+    path, _ = small_pb
+    with pytest.raises(ValueError, match="model file not found"):
+        cb.Model("/nonexistent/model.pb", 4, 32, 3, 4)
+    empty = os.path.join(os.path.dirname(path), "empty.pb")
+    open(empty, "wb").close()
+    with pytest.raises(ValueError, match="model file invalid"):
+        cb.Model(empty, 4, 32, 3, 4)
+    model = cb.Model(path, 2, 32, 3, 4)
+    ids = np.zeros((3, 32), np.int32)
+    m8 = np.ones((3, 32), np.int8)
+    out = np.full((3, 2), 7.0, np.float32)
+    with pytest.raises(ValueError, match="batch_size > max_batch_size"):
+        model.compute(ids, m8, m8, out)
+    with pytest.raises(ValueError, match="invalid output type"):
+        model.compute(ids[:1], m8[:1], m8[:1], out, 17)
+    # batch_size == 0 is a silent no-op
+    model.compute(ids[:0], m8[:0], m8[:0], out)
+    assert (out == 7.0).all()
+    model.close()
+
+
+def test_concurrent_callers_share_one_model(cb, small_pb):
+    """cuBERT_compute is thread-safe per handle (one mutex per replica held for compute + copy-out)."""
+    import threading
+    from cubert_amd.testing import random_inputs
+    path, w = small_pb
+    model = cb.Model(path, 4, 32, 3, 4)
+    cases = [random_inputs(seed=20 + i, batch=1 + i % 4, seq_length=32, vocab=SMALL["vocab"], min_valid=2)
+             for i in range(8)]
+    wants = [oracle.bert_forward(w, *c, 3, 4)["logits"] for c in cases]
+    errors = []
+
+    def worker(i):
+        try:
+            for _ in range(5):
+                out = np.zeros(wants[i].shape, np.float32)
+                model.compute(*cases[i], out)
+                assert_close(out, wants[i], FP32_TOL, "thread %d" % i)
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(8)]
+    [t.start() for t in threads]
+    [t.join() for t in threads]
+    model.close()
+    assert not errors, errors
