@@ -49,6 +49,8 @@ def main():
     ap.add_argument("--workload", default="C1")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--all-kernels", action="store_true", help="time every kernel kind in an extra untimed pass")
+    ap.add_argument("--device-only", action="store_true",
+                    help="only the device-resident steps (no host-path / batch-1 latency loops): for profiler runs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (replicas on several GPUs share nothing); "
@@ -108,30 +110,32 @@ def main():
         bert.profile([])
 
     # ---- the public path: host arrays in, host array out (PCIe-inclusive), and p50 latency at batch 1
-    out = np.empty((B, m["hidden"]), np.float16 if half else np.float32)
-    o = cubert_amd.Output(out, cubert_amd.OutputType.POOLED_OUTPUT)
-    lat = []
-    for i in range(10 + 30):
-        t = time.perf_counter()
-        bert.compute(ids, mask, seg)
-        bert.output(B, o)
-        if i >= 10:
-            lat.append((time.perf_counter() - t) * 1e3)
-    host_path = {"mean_ms": round(float(np.mean(lat)), 3), "p50_ms": round(float(np.median(lat)), 3),
-                 "sequences_per_s": round(B / (np.mean(lat) * 1e-3), 1), "output": "POOLED_OUTPUT"}
-    lat1 = []
-    for i in range(20 + 100):
-        t = time.perf_counter()
-        bert.compute(ids[:1], mask[:1], seg[:1])
-        bert.output(1, o)
-        if i >= 20:
-            lat1.append((time.perf_counter() - t) * 1e3)
-    p50_b1 = round(float(np.median(lat1)), 3)
+    host_path, p50_b1 = None, None
+    if not args.device_only:
+        out = np.empty((B, m["hidden"]), np.float16 if half else np.float32)
+        o = cubert_amd.Output(out, cubert_amd.OutputType.POOLED_OUTPUT)
+        lat = []
+        for i in range(10 + 30):
+            t = time.perf_counter()
+            bert.compute(ids, mask, seg)
+            bert.output(B, o)
+            if i >= 10:
+                lat.append((time.perf_counter() - t) * 1e3)
+        host_path = {"mean_ms": round(float(np.mean(lat)), 3), "p50_ms": round(float(np.median(lat)), 3),
+                     "sequences_per_s": round(B / (np.mean(lat) * 1e-3), 1), "output": "POOLED_OUTPUT"}
+        lat1 = []
+        for i in range(20 + 100):
+            t = time.perf_counter()
+            bert.compute(ids[:1], mask[:1], seg[:1])
+            bert.output(1, o)
+            if i >= 20:
+                lat1.append((time.perf_counter() - t) * 1e3)
+        p50_b1 = round(float(np.median(lat1)), 3)
     bert.close()
 
     # ---- CPU baseline: the oracle (a port of the reference's CPU path) on this host's cores
     cpu = None
-    if not args.no_cpu:
+    if not args.no_cpu and not args.device_only:
         import oracle
         threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
         oracle.lib()

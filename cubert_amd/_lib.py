@@ -69,6 +69,7 @@ SIGNATURES = {
     "cubert_event_destroy": (ci, [vp]),
     "cubert_event_record": (ci, [vp, vp]),
     "cubert_event_elapsed_ms": (ci, [vp, vp, ctypes.POINTER(cf)]),
+    "cubert_time_next_launch": (ci, [vp, vp]),
     "cubert_blas_create": (vp, []),
     "cubert_blas_destroy": (ci, [vp]),
     "cubert_blas_set_stream": (ci, [vp, vp]),

@@ -42,15 +42,24 @@ public:
 
     bool on(Kind k) const { return (mask >> k) & 1u; }
 
+    // The layer kernels (kinds 0..6) are one launch each: the launch itself carries the event pair and
+    // the elapsed time is the kernel's execution time.  GEMM kinds may be several library launches, so
+    // they are bracketed by marker events (which adds the gaps between launches).
+    static bool single_launch(Kind k) { return k < kDenseGemm; }
+
     void begin(Kind k, void *stream) {
         if (!on(k)) return;
         if (used == pool.size()) grow(pool.size() + 1024);
-        CUBERT_CHECK(cubert_event_record(pool[used].first, stream));
+        if (single_launch(k)) {
+            CUBERT_CHECK(cubert_time_next_launch(pool[used].first, pool[used].second));
+        } else {
+            CUBERT_CHECK(cubert_event_record(pool[used].first, stream));
+        }
     }
 
     void end(Kind k, void *stream) {
         if (!on(k)) return;
-        CUBERT_CHECK(cubert_event_record(pool[used].second, stream));
+        if (!single_launch(k)) CUBERT_CHECK(cubert_event_record(pool[used].second, stream));
         kinds_used.push_back(k);
         ++used;
     }

@@ -2,6 +2,7 @@
 // storage <-> fp32 conversion and cross-lane reductions for 64-wide wavefronts.
 #pragma once
 
+#include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -92,6 +93,31 @@ __device__ __forceinline__ int wave_in_block() {
 
 __host__ __device__ __forceinline__ bool is_aligned(const void *p, size_t bytes) {
     return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0;
+}
+
+// ---- launching ------------------------------------------------------------
+// A caller may ask (cubert_time_next_launch) for the next kernel launched from
+// its thread to carry a pair of events that receive the kernel's own start and
+// stop timestamps (the dispatch packet's, not those of separate marker packets
+// around it), so a single launch inside a forward pass can be timed exactly.
+
+struct LaunchTiming {
+    hipEvent_t start = nullptr;
+    hipEvent_t stop = nullptr;
+};
+LaunchTiming &pending_launch_timing();  // thread-local; defined in runtime.hip
+
+template <typename... Params, typename... Args>
+inline int launch(void (*kernel)(Params...), dim3 grid, dim3 block, hipStream_t stream, Args... args) {
+    LaunchTiming &t = pending_launch_timing();
+    if (t.start != nullptr) {
+        hipExtLaunchKernelGGL(kernel, grid, block, 0, stream, t.start, t.stop, 0, static_cast<Params>(args)...);
+        t = LaunchTiming();
+    } else {
+        hipLaunchKernelGGL(kernel, grid, block, 0, stream, static_cast<Params>(args)...);
+    }
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : (int) e;
 }
 
 }  // namespace cubert

@@ -184,11 +184,6 @@ __global__ __launch_bounds__(kBlock) void ln_generic_kernel(T *__restrict__ inou
     }
 }
 
-inline int launch_status() {
-    hipError_t e = hipGetLastError();
-    return e == hipSuccess ? 0 : (int) e;
-}
-
 template <typename T>
 bool vector_ok(int hidden, int vec, std::initializer_list<const void *> ptrs) {
     if (hidden % (kWave * vec) != 0) return false;
@@ -209,12 +204,10 @@ int bias_res_ln(T *inout, const T *residual, const T *bias, const T *beta, const
 #define CUBERT_LN_CASE(VEC, CHUNKS)                                                                      \
     if (hidden == kWave * VEC * CHUNKS && vector_ok<T>(hidden, VEC, {inout, residual, bias, beta, gamma})) { \
         if (bias != nullptr)                                                                             \
-            hipLaunchKernelGGL((bias_res_ln_kernel<T, VEC, CHUNKS, true>), grid, block, 0, s, inout, residual, bias, \
-                               beta, gamma, rows);                                                       \
-        else                                                                                             \
-            hipLaunchKernelGGL((bias_res_ln_kernel<T, VEC, CHUNKS, false>), grid, block, 0, s, inout, residual, bias, \
-                               beta, gamma, rows);                                                       \
-        return launch_status();                                                                          \
+            return launch(bias_res_ln_kernel<T, VEC, CHUNKS, true>, grid, block, s, inout, residual, bias, beta, gamma, \
+                          rows);                                                                         \
+        return launch(bias_res_ln_kernel<T, VEC, CHUNKS, false>, grid, block, s, inout, residual, bias, beta, gamma, \
+                      rows);                                                                             \
     }
     CUBERT_LN_CASE(V, 1)
     CUBERT_LN_CASE(V, 2)
@@ -228,9 +221,8 @@ int bias_res_ln(T *inout, const T *residual, const T *bias, const T *beta, const
     CUBERT_LN_CASE(V, 6)
     CUBERT_LN_CASE(V, 8)
 #undef CUBERT_LN_CASE
-    hipLaunchKernelGGL((ln_generic_kernel<T, false>), grid, block, 0, s, inout, residual, bias, nullptr, nullptr,
-                       nullptr, nullptr, nullptr, beta, gamma, rows, hidden, 1);
-    return launch_status();
+    return launch(ln_generic_kernel<T, false>, grid, block, s, inout, residual, bias, nullptr, nullptr, nullptr, nullptr,
+                  nullptr, beta, gamma, rows, hidden, 1);
 }
 
 template <typename T>
@@ -248,9 +240,8 @@ int embed_ln(const int32_t *ids, const int8_t *segments, const T *word, const T 
     constexpr int V = MaxVec<T>::value;
 #define CUBERT_EMB_CASE(VEC, CHUNKS)                                                                       \
     if (hidden == kWave * VEC * CHUNKS && vector_ok<T>(hidden, VEC, {word, pos, type, beta, gamma, out})) { \
-        hipLaunchKernelGGL((embed_ln_kernel<T, VEC, CHUNKS>), grid, block, 0, s, ids, segments, word, pos, type, \
-                           beta, gamma, out, rows, seq_length);                                            \
-        return launch_status();                                                                            \
+        return launch(embed_ln_kernel<T, VEC, CHUNKS>, grid, block, s, ids, segments, word, pos, type, beta, gamma, \
+                      out, rows, seq_length);                                                              \
     }
     CUBERT_EMB_CASE(V, 1)
     CUBERT_EMB_CASE(V, 2)
@@ -264,9 +255,8 @@ int embed_ln(const int32_t *ids, const int8_t *segments, const T *word, const T 
     CUBERT_EMB_CASE(V, 6)
     CUBERT_EMB_CASE(V, 8)
 #undef CUBERT_EMB_CASE
-    hipLaunchKernelGGL((ln_generic_kernel<T, true>), grid, block, 0, s, out, nullptr, nullptr, ids, segments, word,
-                       pos, type, beta, gamma, rows, hidden, seq_length);
-    return launch_status();
+    return launch(ln_generic_kernel<T, true>, grid, block, s, out, nullptr, nullptr, ids, segments, word, pos, type,
+                  beta, gamma, rows, hidden, seq_length);
 }
 
 }  // namespace

@@ -149,18 +149,11 @@ __global__ __launch_bounds__(kBlock) void softmax_tiny_kernel(const T *__restric
     for (int j = 0; j < channel; ++j) y[j] = from_f32<T>(normalise<T>(__expf(to_f32(x[j]) - mx), sum, inv));
 }
 
-inline int launch_status() {
-    hipError_t e = hipGetLastError();
-    return e == hipSuccess ? 0 : (int) e;
-}
-
 template <typename T, int VEC, int LPR, int CH, int RPG>
 int launch_fast(T *scores, const int8_t *mask, float scale, int batch, int rows_per_batch, hipStream_t s) {
     constexpr int rows_per_block = (kBlock / LPR) * RPG;
     dim3 grid((rows_per_batch + rows_per_block - 1) / rows_per_block, batch), block(kBlock);
-    hipLaunchKernelGGL((mask_scale_softmax_kernel<T, VEC, LPR, CH, RPG>), grid, block, 0, s, scores, mask, scale,
-                       rows_per_batch);
-    return launch_status();
+    return launch(mask_scale_softmax_kernel<T, VEC, LPR, CH, RPG>, grid, block, s, scores, mask, scale, rows_per_batch);
 }
 
 template <typename T>
@@ -202,9 +195,8 @@ int mask_scale_softmax(T *scores, const int8_t *mask, float scale, int batch, in
     }
     const int rows = (int) rows_ll;
     dim3 grid((rows + 3) / 4), block(kBlock);
-    hipLaunchKernelGGL((softmax_generic_kernel<T>), grid, block, 0, s, (const T *) scores, scores, mask, scale, rows,
-                       seq, mask ? rpb : 0);
-    return launch_status();
+    return launch(softmax_generic_kernel<T>, grid, block, s, (const T *) scores, scores, mask, scale, rows, seq,
+                  mask ? rpb : 0);
 }
 
 template <typename T>
@@ -214,13 +206,10 @@ int row_softmax(const T *in, T *out, int rows, int channel, void *stream) {
     hipStream_t s = (hipStream_t) stream;
     if (channel <= 16) {
         dim3 grid((rows + kBlock - 1) / kBlock), block(kBlock);
-        hipLaunchKernelGGL((softmax_tiny_kernel<T>), grid, block, 0, s, in, out, rows, channel);
-    } else {
-        dim3 grid((rows + 3) / 4), block(kBlock);
-        hipLaunchKernelGGL((softmax_generic_kernel<T>), grid, block, 0, s, in, out, (const int8_t *) nullptr, 1.0f,
-                           rows, channel, 0);
+        return launch(softmax_tiny_kernel<T>, grid, block, s, in, out, rows, channel);
     }
-    return launch_status();
+    dim3 grid((rows + 3) / 4), block(kBlock);
+    return launch(softmax_generic_kernel<T>, grid, block, s, in, out, (const int8_t *) nullptr, 1.0f, rows, channel, 0);
 }
 
 }  // namespace

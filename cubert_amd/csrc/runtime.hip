@@ -19,6 +19,14 @@
 #include <vector>
 
 #include "cubert_kernels.h"
+#include "device_common.h"
+
+namespace cubert {
+LaunchTiming &pending_launch_timing() {
+    static thread_local LaunchTiming pending;
+    return pending;
+}
+}  // namespace cubert
 
 namespace {
 
@@ -278,14 +286,23 @@ int cubert_stream_destroy(void *stream) { return stream ? hip_rc(hipStreamDestro
 int cubert_stream_synchronize(void *stream) { return hip_rc(hipStreamSynchronize((hipStream_t) stream)); }
 
 void *cubert_event_create(void) {
+    // Device-scope release: recording the event does not write the caches back to memory, which keeps
+    // the marker cheap and leaves the cache state of the timed kernels as it would be without timing.
     hipEvent_t e = nullptr;
-    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    if (hipEventCreateWithFlags(&e, hipEventReleaseToDevice) != hipSuccess) return nullptr;
     return e;
 }
 
 int cubert_event_destroy(void *event) { return event ? hip_rc(hipEventDestroy((hipEvent_t) event)) : 0; }
 
 int cubert_event_record(void *event, void *stream) { return hip_rc(hipEventRecord((hipEvent_t) event, (hipStream_t) stream)); }
+
+int cubert_time_next_launch(void *start_event, void *stop_event) {
+    cubert::LaunchTiming &t = cubert::pending_launch_timing();
+    t.start = (hipEvent_t) start_event;
+    t.stop = (hipEvent_t) stop_event;
+    return 0;
+}
 
 int cubert_event_elapsed_ms(void *start, void *stop, float *ms) {
     return hip_rc(hipEventElapsedTime(ms, (hipEvent_t) start, (hipEvent_t) stop));

@@ -129,6 +129,10 @@ void *cubert_event_create(void);
 int cubert_event_destroy(void *event);
 int cubert_event_record(void *event, void *stream);
 int cubert_event_elapsed_ms(void *start, void *stop, float *ms); /* both events must have completed */
+/* The next layer kernel launched from the calling thread writes its own start and stop timestamps into the
+ * two events (the kernel's dispatch packet carries them), so cubert_event_elapsed_ms(start, stop) is that
+ * kernel's execution time alone.  One shot: cleared by the launch.  NULL, NULL cancels. */
+int cubert_time_next_launch(void *start_event, void *stop_event);
 
 /* A BLAS context: a hipBLASLt handle, a workspace, a plan cache, bound to one stream. */
 void *cubert_blas_create(void);
