@@ -140,6 +140,95 @@ __global__ __launch_bounds__(kBlock) void embed_ln_kernel(const int32_t *__restr
     ln_finish<T, VEC, CHUNKS>(x, sum, sumsq, g, be, out + (size_t) row * H, lane);
 }
 
+// ---- rows of 96 * VEC elements (768 halves, 384 floats): 1.5 wavefront-wide 16-byte vectors ----
+// Padding such a row to two loads per lane would leave a quarter of the lanes idle, and splitting
+// it into three 8-byte loads doubles the number of memory instructions.  Instead a wavefront takes
+// TWO consecutive rows (3072 bytes) as three full 16-byte loads: load 0 is row 0, load 2 is row 1,
+// load 1 is row 0 in lanes 0..31 and row 1 in lanes 32..63.  Each row still gets its own statistics
+// (four wavefront reductions instead of two).  An odd last row is handled with the second row masked.
+template <typename T, int VEC, bool EMBED, bool HAS_BIAS>
+__global__ __launch_bounds__(kBlock) void ln_pair_kernel(T *__restrict__ inout, const T *__restrict__ residual,
+                                                         const T *__restrict__ bias, const int32_t *__restrict__ ids,
+                                                         const int8_t *__restrict__ segments,
+                                                         const T *__restrict__ word, const T *__restrict__ pos,
+                                                         const T *__restrict__ type, const T *__restrict__ beta,
+                                                         const T *__restrict__ gamma, int rows, int seq_length) {
+    constexpr int H = 96 * VEC;
+    const int row0 = (blockIdx.x * kRowsPerBlock + wave_in_block()) * 2;
+    if (row0 >= rows) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const bool has_second = row0 + 1 < rows;  // wavefront-uniform
+    const bool upper = lane >= 32;            // in load 1 the upper half of the lanes belongs to the second row
+
+    // wavefront-uniform row bases (scalar loads for the ids)
+    const T *src_a[2], *src_b[2], *src_c[2];
+    if (EMBED) {
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const int row = (k == 1 && !has_second) ? row0 : row0 + k;
+            src_a[k] = word + (size_t) ids[row] * H;
+            src_b[k] = pos + (size_t) (row % seq_length) * H;
+            src_c[k] = type + (size_t) segments[row] * H;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            src_a[k] = inout + (size_t) (row0 + k) * H;
+            src_b[k] = bias;
+            src_c[k] = residual + (size_t) (row0 + k) * H;
+        }
+    }
+    T *dst[2] = {inout + (size_t) row0 * H, inout + (size_t) (row0 + 1) * H};
+
+    Vec<T, VEC> a[3], b[3], c[3], g[3], be[3];
+    int col[3];
+    bool second[3], active[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        const int flat = (k * kWave + lane) * VEC;  // element offset inside the two-row span
+        second[k] = k == 2 || (k == 1 && upper);
+        col[k] = second[k] ? flat - H : flat;
+        active[k] = !second[k] || has_second;
+        const Vec<T, VEC> zero = {};
+        a[k] = active[k] ? load_vec<T, VEC>((second[k] ? src_a[1] : src_a[0]) + col[k]) : zero;
+        c[k] = active[k] ? load_vec<T, VEC>((second[k] ? src_c[1] : src_c[0]) + col[k]) : zero;
+        if (EMBED) b[k] = active[k] ? load_vec<T, VEC>((second[k] ? src_b[1] : src_b[0]) + col[k]) : zero;
+    }
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        if (!EMBED && HAS_BIAS) b[k] = load_vec<T, VEC>(bias + col[k]);
+        g[k] = load_vec<T, VEC>(gamma + col[k]);
+        be[k] = load_vec<T, VEC>(beta + col[k]);
+    }
+    float x[3][VEC], s[3], ss[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        s[k] = 0.f;
+        ss[k] = 0.f;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            float v = to_f32(a[k].v[i]);
+            if (EMBED || HAS_BIAS) v += to_f32(b[k].v[i]);  // (word + position) or (gemm output + bias) first
+            v += to_f32(c[k].v[i]);
+            x[k][i] = v;
+            s[k] += v;
+            ss[k] += v * v;
+        }
+    }
+    float mean[2], rstd[2];
+    ln_stats(s[0] + (upper ? 0.f : s[1]), ss[0] + (upper ? 0.f : ss[1]), H, mean[0], rstd[0]);
+    ln_stats(s[2] + (upper ? s[1] : 0.f), ss[2] + (upper ? ss[1] : 0.f), H, mean[1], rstd[1]);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        const float m = second[k] ? mean[1] : mean[0];
+        const float r = second[k] ? rstd[1] : rstd[0];
+        Vec<T, VEC> o;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) o.v[i] = from_f32<T>(to_f32(be[k].v[i]) + (to_f32(g[k].v[i]) * r) * (x[k][i] - m));
+        if (active[k]) store_vec<T, VEC>((second[k] ? dst[1] : dst[0]) + col[k], o);
+    }
+}
+
 // ---- generic path: any hidden size, scalar accesses, operands read twice ----
 
 template <typename T, bool EMBED>
@@ -201,6 +290,14 @@ int bias_res_ln(T *inout, const T *residual, const T *bias, const T *beta, const
     hipStream_t s = (hipStream_t) stream;
     dim3 grid((rows + kRowsPerBlock - 1) / kRowsPerBlock), block(kBlock);
     constexpr int V = MaxVec<T>::value;  // 4 floats or 8 halves
+    if (hidden == 96 * V && vector_ok<T>(2 * kWave * V, V, {inout, residual, bias, beta, gamma})) {
+        dim3 pair_grid(((rows + 1) / 2 + kRowsPerBlock - 1) / kRowsPerBlock);
+        if (bias != nullptr)
+            return launch(ln_pair_kernel<T, V, false, true>, pair_grid, block, s, inout, residual, bias, nullptr, nullptr,
+                          nullptr, nullptr, nullptr, beta, gamma, rows, 1);
+        return launch(ln_pair_kernel<T, V, false, false>, pair_grid, block, s, inout, residual, bias, nullptr, nullptr,
+                      nullptr, nullptr, nullptr, beta, gamma, rows, 1);
+    }
 #define CUBERT_LN_CASE(VEC, CHUNKS)                                                                      \
     if (hidden == kWave * VEC * CHUNKS && vector_ok<T>(hidden, VEC, {inout, residual, bias, beta, gamma})) { \
         if (bias != nullptr)                                                                             \
@@ -238,6 +335,11 @@ int embed_ln(const int32_t *ids, const int8_t *segments, const T *word, const T 
     hipStream_t s = (hipStream_t) stream;
     dim3 grid((rows + kRowsPerBlock - 1) / kRowsPerBlock), block(kBlock);
     constexpr int V = MaxVec<T>::value;
+    if (hidden == 96 * V && vector_ok<T>(2 * kWave * V, V, {word, pos, type, beta, gamma, out})) {
+        dim3 pair_grid(((rows + 1) / 2 + kRowsPerBlock - 1) / kRowsPerBlock);
+        return launch(ln_pair_kernel<T, V, true, false>, pair_grid, block, s, out, nullptr, nullptr, ids, segments, word,
+                      pos, type, beta, gamma, rows, seq_length);
+    }
 #define CUBERT_EMB_CASE(VEC, CHUNKS)                                                                       \
     if (hidden == kWave * VEC * CHUNKS && vector_ok<T>(hidden, VEC, {word, pos, type, beta, gamma, out})) { \
         return launch(embed_ln_kernel<T, VEC, CHUNKS>, grid, block, s, ids, segments, word, pos, type, beta, gamma, \

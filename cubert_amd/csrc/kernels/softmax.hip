@@ -14,7 +14,9 @@
 //
 // A row of seq elements is spread over LPR lanes (a power of two <= 64), each
 // holding CH vectors of VEC elements, so short rows pack several to a
-// wavefront: seq=32 fp32 -> 8 lanes per row, 8 rows per wavefront.
+// wavefront: seq=32 fp32 -> 8 lanes per row, 8 rows per wavefront.  The mask
+// bytes of a lane's columns are re-read per row (seq bytes per batch element,
+// L1 resident).
 
 #include "cubert_kernels.h"
 #include "device_common.h"
@@ -31,73 +33,60 @@ __device__ __forceinline__ float normalise<float>(float e, float sum, float) { r
 template <>
 __device__ __forceinline__ float normalise<half_t>(float e, float, float inv_sum) { return e * inv_sum; }
 
-// grid.x: blocks of rows inside one batch element, grid.y: batch element.
-template <typename T, int VEC, int LPR, int CH, int RPG>
-__global__ __launch_bounds__(kBlock) void mask_scale_softmax_kernel(T *__restrict__ scores,
-                                                                    const int8_t *__restrict__ mask, float scale,
-                                                                    int rows_per_batch) {
+// grid.x: blocks of rows inside one batch element, grid.y: batch element.  Every lane group
+// handles one row (one or a few 16-byte loads per lane) and a workgroup is a single wavefront:
+// the smallest unit of work per workgroup measured fastest inside the forward pass (64 threads
+// vs 256: 108 vs 117 us at batch 64, seq 512; 40.9 vs 44.6 us at batch 256, seq 128).
+template <typename T, int VEC, int LPR, int CH, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void mask_scale_softmax_kernel(T *__restrict__ scores,
+                                                                   const int8_t *__restrict__ mask, float scale,
+                                                                   int rows_per_batch) {
     constexpr int S = VEC * LPR * CH;
-    constexpr int kGroups = kBlock / LPR;
+    constexpr int kGroups = BLOCK / LPR;
     const int group = threadIdx.x / LPR;
     const int gl = threadIdx.x % LPR;
     const int b = blockIdx.y;
-    const int row0 = (blockIdx.x * kGroups + group) * RPG;
-    T *base = scores + ((size_t) b * rows_per_batch) * S;
+    const int row = blockIdx.x * kGroups + group;
+    if (row >= rows_per_batch) return;  // whole lane groups leave together
+    T *p = scores + ((size_t) b * rows_per_batch + row) * S;
 
-    float addend[CH][VEC];
+    Vec<T, VEC> raw[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) raw[c] = load_vec<T, VEC>(p + (c * LPR + gl) * VEC);
+
+    float x[CH][VEC];
+    float mx = -3.402823466e+38f;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-        const int col = (c * LPR + gl) * VEC;
         if (mask != nullptr) {
-            Vec<int8_t, VEC> m = load_vec<int8_t, VEC>(mask + (size_t) b * S + col);
+            Vec<int8_t, VEC> m = load_vec<int8_t, VEC>(mask + (size_t) b * S + (c * LPR + gl) * VEC);
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) addend[c][i] = m.v[i] ? 0.f : kMaskedScore;
+            for (int i = 0; i < VEC; ++i) x[c][i] = to_f32(raw[c].v[i]) * scale + (m.v[i] ? 0.f : kMaskedScore);
         } else {
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) addend[c][i] = 0.f;
+            for (int i = 0; i < VEC; ++i) x[c][i] = to_f32(raw[c].v[i]) * scale;
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) mx = fmaxf(mx, x[c][i]);
+    }
+    mx = group_reduce<LPR>(mx, MaxOp());
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            x[c][i] = __expf(x[c][i] - mx);
+            sum += x[c][i];
         }
     }
-
-    Vec<T, VEC> raw[RPG][CH];
+    sum = group_reduce<LPR>(sum, SumOp());
+    const float inv = 1.f / sum;
 #pragma unroll
-    for (int r = 0; r < RPG; ++r) {
-        if (row0 + r < rows_per_batch) {
+    for (int c = 0; c < CH; ++c) {
+        Vec<T, VEC> o;
 #pragma unroll
-            for (int c = 0; c < CH; ++c) raw[r][c] = load_vec<T, VEC>(base + (size_t) (row0 + r) * S + (c * LPR + gl) * VEC);
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < RPG; ++r) {
-        if (row0 + r >= rows_per_batch) continue;  // whole lane groups leave together
-        float x[CH][VEC];
-        float mx = -3.402823466e+38f;
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                x[c][i] = to_f32(raw[r][c].v[i]) * scale + addend[c][i];
-                mx = fmaxf(mx, x[c][i]);
-            }
-        }
-        mx = group_reduce<LPR>(mx, MaxOp());
-        float sum = 0.f;
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                x[c][i] = __expf(x[c][i] - mx);
-                sum += x[c][i];
-            }
-        }
-        sum = group_reduce<LPR>(sum, SumOp());
-        const float inv = 1.f / sum;
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            Vec<T, VEC> o;
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) o.v[i] = from_f32<T>(normalise<T>(x[c][i], sum, inv));
-            store_vec<T, VEC>(base + (size_t) (row0 + r) * S + (c * LPR + gl) * VEC, o);
-        }
+        for (int i = 0; i < VEC; ++i) o.v[i] = from_f32<T>(normalise<T>(x[c][i], sum, inv));
+        store_vec<T, VEC>(p + (c * LPR + gl) * VEC, o);
     }
 }
 
@@ -149,11 +138,13 @@ __global__ __launch_bounds__(kBlock) void softmax_tiny_kernel(const T *__restric
     for (int j = 0; j < channel; ++j) y[j] = from_f32<T>(normalise<T>(__expf(to_f32(x[j]) - mx), sum, inv));
 }
 
-template <typename T, int VEC, int LPR, int CH, int RPG>
+template <typename T, int VEC, int LPR, int CH>
 int launch_fast(T *scores, const int8_t *mask, float scale, int batch, int rows_per_batch, hipStream_t s) {
-    constexpr int rows_per_block = (kBlock / LPR) * RPG;
-    dim3 grid((rows_per_batch + rows_per_block - 1) / rows_per_block, batch), block(kBlock);
-    return launch(mask_scale_softmax_kernel<T, VEC, LPR, CH, RPG>, grid, block, s, scores, mask, scale, rows_per_batch);
+    constexpr int kThreads = kWave;
+    constexpr int rows_per_block = kThreads / LPR;
+    dim3 grid((rows_per_batch + rows_per_block - 1) / rows_per_block, batch), block(kThreads);
+    return launch(mask_scale_softmax_kernel<T, VEC, LPR, CH, kThreads>, grid, block, s, scores, mask, scale,
+                  rows_per_batch);
 }
 
 template <typename T>
@@ -167,28 +158,23 @@ int mask_scale_softmax(T *scores, const int8_t *mask, float scale, int batch, in
     constexpr int V = MaxVec<T>::value;
     const bool aligned = is_aligned(scores, 16) && (mask == nullptr || is_aligned(mask, V)) && seq % V == 0;
     if (aligned) {
-        // Several rows per lane group amortise the mask read and deepen the load queue, but only
-        // pay once the grid still has a few workgroups for each of the 256 compute units.
-        const bool big = rows_ll * seq * (long long) sizeof(T) >= (32LL << 20);
-#define CUBERT_SM_CASE(NVEC, LPR, CH, RPG)                                                   \
-    case NVEC:                                                                               \
-        return big ? launch_fast<T, V, LPR, CH, RPG>(scores, mask, scale, batch, rpb, s)     \
-                   : launch_fast<T, V, LPR, CH, 1>(scores, mask, scale, batch, rpb, s);
+#define CUBERT_SM_CASE(NVEC, LPR, CH) \
+    case NVEC: return launch_fast<T, V, LPR, CH>(scores, mask, scale, batch, rpb, s);
         switch (seq / V) {  // vectors per row
-            CUBERT_SM_CASE(1, 1, 1, 4)
-            CUBERT_SM_CASE(2, 2, 1, 4)
-            CUBERT_SM_CASE(4, 4, 1, 4)
-            CUBERT_SM_CASE(8, 8, 1, 4)
-            CUBERT_SM_CASE(16, 16, 1, 4)
-            CUBERT_SM_CASE(32, 32, 1, 2)
-            CUBERT_SM_CASE(64, 64, 1, 2)
-            CUBERT_SM_CASE(128, 64, 2, 1)
-            CUBERT_SM_CASE(256, 64, 4, 1)
-            CUBERT_SM_CASE(12, 4, 3, 4)
-            CUBERT_SM_CASE(24, 8, 3, 4)
-            CUBERT_SM_CASE(48, 16, 3, 2)   // seq 384 in fp16
-            CUBERT_SM_CASE(96, 32, 3, 2)   // seq 384 in fp32
-            CUBERT_SM_CASE(192, 64, 3, 1)
+            CUBERT_SM_CASE(1, 1, 1)
+            CUBERT_SM_CASE(2, 2, 1)
+            CUBERT_SM_CASE(4, 4, 1)
+            CUBERT_SM_CASE(8, 8, 1)
+            CUBERT_SM_CASE(16, 16, 1)
+            CUBERT_SM_CASE(32, 32, 1)
+            CUBERT_SM_CASE(64, 64, 1)
+            CUBERT_SM_CASE(128, 64, 2)
+            CUBERT_SM_CASE(256, 64, 4)
+            CUBERT_SM_CASE(12, 4, 3)
+            CUBERT_SM_CASE(24, 8, 3)
+            CUBERT_SM_CASE(48, 16, 3)   // seq 384 in fp16
+            CUBERT_SM_CASE(96, 32, 3)   // seq 384 in fp32
+            CUBERT_SM_CASE(192, 64, 3)
             default: break;
         }
 #undef CUBERT_SM_CASE

@@ -175,7 +175,7 @@ def test_batch_matmul_reference_vectors(K, case):
 
 @pytest.mark.parametrize("name", ["f32", "f16"])
 @pytest.mark.parametrize("rows,hidden", [(4096, 768), (1000, 1024), (37, 768), (5, 256), (64, 1280), (3, 6), (9, 100),
-                                         (2, 4096)])
+                                         (2, 4096), (7, 384), (1, 768), (2, 768)])
 @pytest.mark.parametrize("with_bias", [True, False])
 def test_bias_res_ln(K, name, rows, hidden, with_bias):
     rng = np.random.default_rng(rows * 7 + hidden)
@@ -195,7 +195,8 @@ def test_bias_res_ln(K, name, rows, hidden, with_bias):
 
 @pytest.mark.parametrize("name", ["f32", "f16"])
 @pytest.mark.parametrize("batch,seq,hidden,vocab", [(128, 32, 768, 21128), (3, 128, 1024, 3000), (2, 4, 6, 11),
-                                                    (1, 512, 768, 21128), (5, 7, 100, 50)])
+                                                    (1, 512, 768, 21128), (5, 7, 100, 50), (5, 7, 768, 50),
+                                                    (3, 3, 384, 20), (1, 1, 768, 9)])
 def test_embed_ln(K, name, batch, seq, hidden, vocab):
     rng = np.random.default_rng(batch + seq + hidden)
     w = {"bert/embeddings/word_embeddings": q(rng.normal(0, 0.02, (vocab, hidden)), name),
