@@ -49,6 +49,9 @@ def main():
     ap.add_argument("--workload", default="C1")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--all-kernels", action="store_true", help="time every kernel kind in an extra untimed pass")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="instead of the model: 10 launches of a plain row copy of known size (100 MB read, 100 MB "
+                         "written), the yardstick for hardware traffic counters")
     ap.add_argument("--device-only", action="store_true",
                     help="only the device-resident steps (no host-path / batch-1 latency loops): for profiler runs")
     args = ap.parse_args()
@@ -59,6 +62,20 @@ def main():
 
     import cubert_amd
     from cubert_amd.testing import CONFIGS, config_inputs, config_weights
+
+    if args.calibrate_copy:
+        import torch
+        from cubert_amd import kernels
+        rows, width = 32768, 768
+        table = torch.randn(rows, width, device="cuda")
+        ids = torch.arange(rows, dtype=torch.int32, device="cuda")
+        for _ in range(10):
+            out = kernels.gather(ids, table)
+        torch.cuda.synchronize()
+        assert torch.equal(out, table)
+        print(json.dumps({"copy_kernel": "gather_kernel<float, int, 4>", "bytes_read": rows * width * 4 + rows * 4,
+                          "bytes_written": rows * width * 4, "launches": 10}))
+        return
 
     cfg = CONFIGS[args.workload]
     m = cfg["model"]
@@ -88,11 +105,18 @@ def main():
     value = B / (ms_per_step * 1e-3)
 
     alg = algorithmic_bytes(cfg)
+    # HBM-side bytes per launch from hardware counters (a separate profiler run; see profiles/traffic_pmc.md)
+    traffic = None
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic_pmc.json")) as f:
+            traffic = json.load(f)["workloads"][args.workload][dominant]["total"]
+    except (OSError, KeyError, ValueError):
+        pass
     total_ms, launches = prof[dominant]
     avg_us = total_ms * 1e3 / launches
     achieved = alg[dominant] / (avg_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "algorithmic_bytes_per_launch": alg[dominant], "avg_launch_us": round(avg_us, 2), "launches": launches}
 
     # ---- every kernel kind, in an extra untimed pass (reported, not part of `value`)
