@@ -84,6 +84,8 @@ for _t in ("f32", "f16"):
         "cubert_bias_gelu_" + _t: (ci, [vp, vp, ci, ci, vp]),
         "cubert_mask_scale_softmax_" + _t: (ci, [vp, vp, cf, ci, ci, ci, vp]),
         "cubert_row_softmax_" + _t: (ci, [vp, vp, ci, ci, vp]),
+        "cubert_attention_scores_" + _t: (ci, [vp, vp, ci, vp, cf, ci, ci, ci, ci, vp]),
+        "cubert_attention_context_" + _t: (ci, [vp, vp, ci, vp, ci, ci, ci, ci, ci, vp]),
         "cubert_bias_tanh_" + _t: (ci, [vp, vp, ci, ci, vp]),
         "cubert_mean_pool_" + _t: (ci, [vp, vp, ci, ci, ci, vp]),
         "cubert_gemm_" + _t: (ci, [vp, ci, ci, ci, ci, ci, cf, vp, ci, vp, ci, cf, vp, ci, vp]),

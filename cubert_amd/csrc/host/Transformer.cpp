@@ -108,8 +108,9 @@ void Transformer<T>::_pre_compute(size_t) {}
 
 // scores[b, a, q, k] = (1/sqrt d) * sum_j Q[b, q, a, j] K[b, k, a, j];  softmax with mask;
 // ctx[b, q, a, :] = sum_k p[b, a, q, k] V[b, k, a, :].   Q, K, V are column blocks of qkv[M, 3H].
-// The (b, a) problems have two strides (b: seq*3H, a: d), a strided-batched GEMM has one, so the
-// shorter of the two axes is looped on the host and the longer one is the GEMM batch.
+// The contractions run as one matrix-core launch each where the shape allows.  Otherwise: the (b, a)
+// problems have two strides (b: seq*3H, a: d), a strided-batched GEMM has one, so the shorter of the two
+// axes is looped on the host and the longer one is the GEMM batch.
 template <typename T>
 void Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *mask) {
     void *stream = cuBERT::blas_get_stream(cublas);
@@ -128,24 +129,28 @@ void Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *ma
     const long long ctx_inner = loop_heads ? (long long) S * H : (long long) d;
 
     {
-    Timed t(profiler, Profiler::kAttentionGemm, stream);
-    for (int o = 0; o < outer; ++o) {
-        // column-major: scores_ba (S_k x S_q, ld S) = K_ba^T (d x S_k, ld 3H)^T * Q_ba (d x S_q, ld 3H)
-        cuBERT::blas_gemm_strided_batch(cublas, true, false, S, S, d, alpha, K + o * in_outer, ld, in_inner,
-                                        Q + o * in_outer, ld, in_inner, 0.f, attention_scores + o * sc_outer, S,
-                                        sc_inner, inner);
-    }
+        Timed t(profiler, Profiler::kAttentionGemm, stream);
+        if (!cuBERT::attention_scores(Q, K, ld, attention_scores, alpha, B, A, S, d, stream)) {
+            for (int o = 0; o < outer; ++o) {
+                // column-major: scores_ba (S_k x S_q, ld S) = K_ba^T (d x S_k, ld 3H)^T * Q_ba (d x S_q, ld 3H)
+                cuBERT::blas_gemm_strided_batch(cublas, true, false, S, S, d, alpha, K + o * in_outer, ld, in_inner,
+                                                Q + o * in_outer, ld, in_inner, 0.f, attention_scores + o * sc_outer,
+                                                S, sc_inner, inner);
+            }
+        }
     }
     {
         Timed t(profiler, Profiler::kMaskScaleSoftmax, stream);
         cuBERT::mask_scale_softmax_(attention_scores, mask, 1.0f, B, A, S, stream);
     }
     Timed t(profiler, Profiler::kAttentionGemm, stream);
-    for (int o = 0; o < outer; ++o) {
-        // column-major: ctx_ba (d x S_q, ld H) = V_ba (d x S_k, ld 3H) * p_ba (S_k x S_q, ld S)
-        cuBERT::blas_gemm_strided_batch(cublas, false, false, d, S, S, 1.f, V + o * in_outer, ld, in_inner,
-                                        attention_scores + o * sc_outer, S, sc_inner, 0.f, context_out + o * ctx_outer,
-                                        H, ctx_inner, inner);
+    if (!cuBERT::attention_context(attention_scores, V, ld, context_out, H, B, A, S, d, stream)) {
+        for (int o = 0; o < outer; ++o) {
+            // column-major: ctx_ba (d x S_q, ld H) = V_ba (d x S_k, ld 3H) * p_ba (S_k x S_q, ld S)
+            cuBERT::blas_gemm_strided_batch(cublas, false, false, d, S, S, 1.f, V + o * in_outer, ld, in_inner,
+                                            attention_scores + o * sc_outer, S, sc_inner, 0.f,
+                                            context_out + o * ctx_outer, H, ctx_inner, inner);
+        }
     }
 }
 

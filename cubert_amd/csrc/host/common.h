@@ -154,6 +154,37 @@ inline void mask_scale_softmax_(half *scores, const int8_t *mask, float scale, i
     CUBERT_CHECK(cubert_mask_scale_softmax_f16(h(scores), mask, scale, batch, heads, seq, stream));
 }
 
+// Att_Q_K / Att_QK_V over every (batch, head) problem in one launch (reference: op_att/BatchMatMul.h:17-74).
+// Return false when the shape has no matrix-core kernel; the caller then loops a strided-batched GEMM.
+inline bool attention_scores(const float *q, const float *k, int ld, float *scores, float alpha, int batch, int heads,
+                             int seq, int head_size, void *stream) {
+    const int rc = cubert_attention_scores_f32(q, k, ld, scores, alpha, batch, heads, seq, head_size, stream);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+inline bool attention_scores(const half *q, const half *k, int ld, half *scores, float alpha, int batch, int heads,
+                             int seq, int head_size, void *stream) {
+    const int rc = cubert_attention_scores_f16(h(q), h(k), ld, h(scores), alpha, batch, heads, seq, head_size, stream);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+inline bool attention_context(const float *probs, const float *v, int ld, float *ctx, int ld_ctx, int batch, int heads,
+                              int seq, int head_size, void *stream) {
+    const int rc = cubert_attention_context_f32(probs, v, ld, ctx, ld_ctx, batch, heads, seq, head_size, stream);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+inline bool attention_context(const half *probs, const half *v, int ld, half *ctx, int ld_ctx, int batch, int heads,
+                              int seq, int head_size, void *stream) {
+    const int rc = cubert_attention_context_f16(h(probs), h(v), ld, h(ctx), ld_ctx, batch, heads, seq, head_size, stream);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+
 // reference: op/Softmax.h:8-14
 inline void softmax_(const float *in, float *out, int rows, int channel, void *stream) {
     CUBERT_CHECK(cubert_row_softmax_f32(in, out, rows, channel, stream));

@@ -108,16 +108,22 @@ struct LaunchTiming {
 LaunchTiming &pending_launch_timing();  // thread-local; defined in runtime.hip
 
 template <typename... Params, typename... Args>
-inline int launch(void (*kernel)(Params...), dim3 grid, dim3 block, hipStream_t stream, Args... args) {
+inline int launch_lds(void (*kernel)(Params...), dim3 grid, dim3 block, unsigned lds_bytes, hipStream_t stream,
+                      Args... args) {
     LaunchTiming &t = pending_launch_timing();
     if (t.start != nullptr) {
-        hipExtLaunchKernelGGL(kernel, grid, block, 0, stream, t.start, t.stop, 0, static_cast<Params>(args)...);
+        hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, t.start, t.stop, 0, static_cast<Params>(args)...);
         t = LaunchTiming();
     } else {
-        hipLaunchKernelGGL(kernel, grid, block, 0, stream, static_cast<Params>(args)...);
+        hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, static_cast<Params>(args)...);
     }
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int) e;
+}
+
+template <typename... Params, typename... Args>
+inline int launch(void (*kernel)(Params...), dim3 grid, dim3 block, hipStream_t stream, Args... args) {
+    return launch_lds(kernel, grid, block, 0u, stream, args...);
 }
 
 }  // namespace cubert

@@ -74,6 +74,35 @@ def mask_scale_softmax_(scores, mask, scale=1.0):
     return scores
 
 
+def attention_scores(qkv, batch, heads, seq, head_size, alpha):
+    """scores[B, A, S, S] = alpha * Q K^T from a packed [B*S, 3*H] projection (Q | K | V column blocks).
+    Returns None when the shape has no matrix-core kernel."""
+    hidden = heads * head_size
+    flat = qkv.view(-1)
+    scores = torch.empty((batch, heads, seq, seq), dtype=qkv.dtype, device=qkv.device)
+    fn = getattr(lib(), "cubert_attention_scores_" + _suffix(qkv))
+    rc = fn(_ptr(flat), _ptr(flat[hidden:]), 3 * hidden, _ptr(scores), float(alpha), batch, heads, seq, head_size,
+            _stream())
+    if rc == -2:
+        return None
+    _check(rc, fn.__name__)
+    return scores
+
+
+def attention_context(probs, qkv, batch, heads, seq, head_size):
+    """ctx[B*S, H] = P V with V the third column block of the packed projection."""
+    hidden = heads * head_size
+    flat = qkv.view(-1)
+    ctx = torch.empty((batch * seq, hidden), dtype=qkv.dtype, device=qkv.device)
+    fn = getattr(lib(), "cubert_attention_context_" + _suffix(qkv))
+    rc = fn(_ptr(probs), _ptr(flat[2 * hidden:]), 3 * hidden, _ptr(ctx), hidden, batch, heads, seq, head_size,
+            _stream())
+    if rc == -2:
+        return None
+    _check(rc, fn.__name__)
+    return ctx
+
+
 def row_softmax(x, out=None):
     out = torch.empty_like(x) if out is None else out
     _call("cubert_row_softmax", x, _ptr(x), _ptr(out), x.shape[0], x.shape[1], _stream())

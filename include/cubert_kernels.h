@@ -32,6 +32,7 @@ extern "C" {
 
 typedef uint16_t cubert_half;
 #define CUBERT_BAD_ARGUMENT (-1)
+#define CUBERT_UNSUPPORTED (-2) /* valid arguments, but no kernel for this shape: the caller takes another route */
 
 /* ------------------------------------------------------------------ kernels */
 
@@ -87,6 +88,24 @@ int cubert_mask_scale_softmax_f32(float *scores, const int8_t *mask, float scale
                                   int seq_length, void *stream);
 int cubert_mask_scale_softmax_f16(cubert_half *scores, const int8_t *mask, float scale, int batch, int heads,
                                   int seq_length, void *stream);
+
+/* The two attention contractions over all (batch, head) problems in one launch each.
+ *   scores[b, a, q, k] = alpha * sum_j Q[b, q, a, j] * K[b, k, a, j]      (scores is [batch, heads, seq, seq])
+ *   ctx[b, q, a, j]    = sum_k P[b, a, q, k] * V[b, k, a, j]              (ctx row stride ld_ctx >= heads*head_size)
+ * q, k, v point at element (0, 0) of their [batch*seq, heads*head_size] views, row stride `ld` elements
+ * (3*hidden for a packed QKV buffer).  Matrix-core kernels, fp32 accumulation.  Supported: seq a multiple of
+ * 32, head_size 32 / 64 / 128, 16-byte aligned pointers, batch*heads <= 65535; anything else returns
+ * CUBERT_UNSUPPORTED and launches nothing (the host classes then loop a strided-batched GEMM).
+ * replaces: Att_Q_K<T>::compute and Att_QK_V<T>::compute (pointer-array batched GEMMs), reference
+ * src/cuBERT/op_att/BatchMatMul.h:17-74 (BatchMatMul.cpp:57-68,129-140); alpha as AttentionSelf.cpp:58-60. */
+int cubert_attention_scores_f32(const float *q, const float *k, int ld, float *scores, float alpha, int batch,
+                                int heads, int seq_length, int head_size, void *stream);
+int cubert_attention_scores_f16(const cubert_half *q, const cubert_half *k, int ld, cubert_half *scores, float alpha,
+                                int batch, int heads, int seq_length, int head_size, void *stream);
+int cubert_attention_context_f32(const float *probs, const float *v, int ld, float *ctx, int ld_ctx, int batch,
+                                 int heads, int seq_length, int head_size, void *stream);
+int cubert_attention_context_f16(const cubert_half *probs, const cubert_half *v, int ld, cubert_half *ctx, int ld_ctx,
+                                 int batch, int heads, int seq_length, int head_size, void *stream);
 
 /* Row softmax of a [rows, channel] matrix, in place or not (classifier probabilities).
  * replaces: softmax_<T>(in, out, rows, channel, sum_buf, stream), reference src/cuBERT/op/Softmax.h:8-14. */

@@ -305,6 +305,44 @@ def test_gather(K, name, idt):
     assert np.array_equal(got, oracle.embedding(ids, table))  # a copy: bit exact
 
 
+# ------------------------------------------------------------------ attention contractions (matrix-core kernels)
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("batch,heads,seq,d", [(3, 12, 32, 64), (2, 4, 128, 64), (1, 2, 512, 64), (2, 3, 64, 32),
+                                               (1, 2, 96, 128), (2, 16, 128, 64), (5, 1, 32, 64), (1, 2, 256, 64)])
+def test_attention_scores_and_context(K, name, batch, heads, seq, d):
+    rng = np.random.default_rng(batch * 1000 + heads * 100 + seq + d)
+    H = heads * d
+    qkv = q(rng.normal(0, 1, (batch * seq, 3 * H)), name)
+    qh, kh, vh = qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:]
+    alpha = 1.0 / math.sqrt(d)
+    dqkv = dev(qkv, tdt(name))
+    scores = K.attention_scores(dqkv, batch, heads, seq, d, alpha)
+    assert scores is not None
+    # the oracle (pinned by the reference's BatchMatMulTest vectors) lays scores out [B, S_q, A, S_k]
+    want = oracle.att_q_k(np.ascontiguousarray(qh), np.ascontiguousarray(kh), batch, seq, heads, d, alpha=alpha)
+    want = want.transpose(0, 2, 1, 3)
+    assert_close(host(scores), want, 2e-5 if name == "f32" else 2e-3, "attention_scores %s" % name)
+    # context from row-stochastic P (what the softmax hands over)
+    p = rng.random((batch, heads, seq, seq)).astype(np.float32)
+    p = q(p / p.sum(-1, keepdims=True), name)
+    ctx = K.attention_context(dev(p, tdt(name)), dqkv, batch, heads, seq, d)
+    assert ctx is not None
+    want_ctx = oracle.att_qk_v(np.ascontiguousarray(p.transpose(0, 2, 1, 3)), np.ascontiguousarray(vh), batch, seq,
+                               heads, d).reshape(batch * seq, H)
+    assert_close(host(ctx), want_ctx, 2e-5 if name == "f32" else 2e-3, "attention_context %s" % name)
+
+
+def test_attention_unsupported_shapes_are_declined(K):
+    """Shapes without a matrix-core kernel return CUBERT_UNSUPPORTED and launch nothing; the host classes then
+    loop the strided-batched GEMM (covered by the encoder reference vectors, seq 4, head size 3)."""
+    qkv = torch.zeros((2 * 4, 3 * 6), device="cuda")
+    assert K.attention_scores(qkv, 2, 2, 4, 3, 1.0) is None
+    assert K.attention_context(torch.zeros((2, 2, 4, 4), device="cuda"), qkv, 2, 2, 4, 3) is None
+    qkv = torch.zeros((2 * 40, 3 * 128), device="cuda")
+    assert K.attention_scores(qkv, 2, 2, 40, 64, 1.0) is None  # seq not a multiple of 32
+
+
 # ------------------------------------------------------------------ GEMM convention
 
 @pytest.mark.parametrize("name", ["f32", "f16"])
