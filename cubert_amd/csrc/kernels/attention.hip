@@ -6,16 +6,20 @@
 // size), which a strided-batched library GEMM cannot express, so the library path needs
 // min(batch, heads) launches per contraction; here a problem is addressed from blockIdx.
 //
-// Both kernels run on the matrix cores: one wavefront accumulates 32x32 tiles with
+// All kernels run on the matrix cores: a wavefront accumulates 32x32 tiles with
 // v_mfma_f32_32x32x16_f16 (fp16 storage) or v_mfma_f32_32x32x2_f32 (fp32 storage), fp32 accumulation.
-// An MFMA sums over its K slots in whatever order the operands name them, as long as A and B agree;
-// lane half hh = lane/32 therefore takes the contiguous half [hh*K/2, (hh+1)*K/2) of the reduction
-// axis, so every operand fetch is a 16-byte load of consecutive elements of one row.
-//   * scores: A = 32 query rows, B = 32 key rows, both straight from global memory (the head slice of a
-//     row is one or two cache lines); no LDS.
-//   * context: A = 32 rows of P from global memory (the big operand, read exactly once), B = V^T, which is
-//     staged transposed in LDS once per workgroup ([head_size][seq + pad]) because an MFMA B operand
-//     needs consecutive k for a fixed column and V is stored with consecutive columns.
+// An MFMA sums over its K slots in whatever order the operands name them, as long as A and B agree,
+// so the two lane halves (hh = lane / 32) are given whatever split of the reduction axis makes their
+// 16-byte operand fetches land where memory likes them.
+//   * scores, seq < 128 (or wide head rows): one wavefront = 32 queries x 32..128 keys, operands straight
+//     from global memory, no LDS.
+//   * scores, seq >= 128: a workgroup owns a 128 x 128 tile; the 128 query rows and 128 key rows of the head
+//     are loaded once with coalesced 16-byte loads (all issued before the first LDS write) and kept in LDS;
+//     each wavefront computes a 64 x 64 sub-tile as 2 x 2 MFMA tiles with A = key rows, B = query rows, so a
+//     lane ends up with 4 consecutive keys of one query; results are staged in LDS and leave as full rows.
+//   * context: A = 32 rows of P from global memory (the big operand, read exactly once), B = V^T, staged
+//     transposed in LDS once per workgroup ([head_size][seq + pad]) because an MFMA B operand needs
+//     consecutive k for a fixed column and V is stored with consecutive columns.
 
 #include <initializer_list>
 
@@ -98,6 +102,106 @@ __global__ __launch_bounds__(kBlock) void attention_scores_kernel(const T *__res
     }
 }
 
+// grid = (ceil(seq / 128) query blocks, ceil(seq / 128) key blocks, batch * heads); 256 threads.
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void attention_scores_tiled_kernel(const T *__restrict__ q,
+                                                                        const T *__restrict__ k, int ld,
+                                                                        T *__restrict__ scores, float alpha, int seq,
+                                                                        int heads) {
+    constexpr int V = Mma<T>::kVec;
+    constexpr int kSteps = D / (2 * V);
+    constexpr int kPitch = D + V;                          // operand row pitch (+16 bytes: conflict-free 16-byte reads)
+    constexpr int kOutPitch = 64 + 8 / (int) sizeof(T);    // staged output row pitch (+8 bytes)
+    constexpr int kOperands = 2 * 128 * kPitch, kStage = 4 * 64 * kOutPitch;
+    __shared__ __align__(16) T lds[kOperands > kStage ? kOperands : kStage];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int r = lane & 31, hh = lane >> 5, wave = wave_in_block();
+    const int bh = blockIdx.z;
+    const int b = bh / heads, h = bh - b * heads;
+    const int q0 = blockIdx.x * 128, k0 = blockIdx.y * 128;
+
+    // rows 0..127 of the staging area are queries, 128..255 keys; rows past the sequence are zero
+    constexpr int kVecPerRow = D / V;
+    constexpr int kLoads = kVecPerRow;  // 256 rows * kVecPerRow vectors / 256 threads
+    Vec<T, V> x[kLoads];
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+        const int idx = threadIdx.x + u * kBlock;
+        const int row = idx / kVecPerRow, c = idx - row * kVecPerRow;
+        const bool is_key = row >= 128;
+        const int src_row = (is_key ? k0 - 128 : q0) + row;
+        x[u] = Vec<T, V>{};
+        if (src_row < seq) {
+            x[u] = load_vec<T, V>((is_key ? k : q) + ((size_t) b * seq + src_row) * ld + (size_t) h * D + c * V);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+        const int idx = threadIdx.x + u * kBlock;
+        const int row = idx / kVecPerRow, c = idx - row * kVecPerRow;
+        store_vec<T, V>(lds + row * kPitch + c * V, x[u]);
+    }
+    __syncthreads();
+
+    const T *s_q = lds, *s_k = lds + 128 * kPitch;
+    const int wq = wave >> 1, wk = wave & 1;
+    v16f32 acc[2][2];  // [key tile][query tile]
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = v16f32{};
+    }
+#pragma unroll
+    for (int t = 0; t < kSteps; ++t) {
+        // reduction slot s of step t in lane half hh is head column t*2V + hh*V + s
+        Vec<T, V> ak[2], bq[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            ak[i] = load_vec<T, V>(s_k + (wk * 64 + i * 32 + r) * kPitch + t * 2 * V + hh * V);
+            bq[i] = load_vec<T, V>(s_q + (wq * 64 + i * 32 + r) * kPitch + t * 2 * V + hh * V);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) Mma<T>::run(acc[i][j], ak[i], bq[j]);
+        }
+    }
+    __syncthreads();  // every wavefront is done with the operands: the space now stages the output
+
+    // lane owns query j*32 + r and, per accumulator group g, keys i*32 + g*8 + hh*4 .. +3
+    T *stage = lds + wave * 64 * kOutPitch;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                Vec<T, 4> o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o.v[e] = from_f32<T>(acc[i][j][g * 4 + e] * alpha);
+                store_vec<T, 4>(stage + (j * 32 + r) * kOutPitch + i * 32 + g * 8 + hh * 4, o);
+            }
+        }
+    }
+    // The same wavefront reads back what it staged; LDS operations of one wavefront complete in order.
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    __builtin_amdgcn_wave_barrier();
+    constexpr int kChunks = 64 / V;        // 16-byte chunks per staged row
+    constexpr int kRowsPerPass = kWave / kChunks;
+    const int chunk = lane % kChunks, row_in = lane / kChunks;
+    const int q_base = q0 + wq * 64, k_base = k0 + wk * 64;
+    if (k_base + chunk * V < seq) {  // seq is a multiple of 32, so a chunk is all inside or all outside
+#pragma unroll
+        for (int pass = 0; pass < 64 / kRowsPerPass; ++pass) {
+            const int row = row_in + kRowsPerPass * pass;
+            if (q_base + row < seq) {
+                store_vec<T, V>(scores + ((size_t) bh * seq + q_base + row) * seq + k_base + chunk * V,
+                                load_vec<T, V>(stage + row * kOutPitch + chunk * V));
+            }
+        }
+    }
+}
+
 // grid = (query-tile groups, batch * heads); dynamic LDS = D * (seq + pad) elements.
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void attention_context_kernel(const T *__restrict__ probs, const T *__restrict__ v,
@@ -106,22 +210,23 @@ __global__ __launch_bounds__(kBlock) void attention_context_kernel(const T *__re
     extern __shared__ __align__(16) unsigned char smem[];
     T *vt = reinterpret_cast<T *>(smem);  // V^T: [D][pitch]
     constexpr int V = Mma<T>::kVec;
-    constexpr int kPad = 16 / sizeof(T);
     constexpr int kColTiles = D / 32;
-    const int pitch = seq + kPad;
+    constexpr int kPrefetch = 4;  // P vectors in flight per lane
+    const int pitch = seq + V;    // +16 bytes: conflict-free 16-byte reads down a column of V^T
     const int lane = threadIdx.x & (kWave - 1);
     const int r = lane & 31, hh = lane >> 5;
     const int bh = blockIdx.y;
     const int b = bh / heads, h = bh - b * heads;
 
-    // stage V[b, :, h, :] transposed: coalesced 16-byte global reads, element-wise LDS writes
+    // Stage V[b, :, h, :] transposed.  A thread takes one head column j and V consecutive keys: V element loads
+    // (consecutive threads = consecutive j: coalesced), one 16-byte LDS write.
     const T *v_head = v + (size_t) b * seq * ld + (size_t) h * D;
-    for (int idx = threadIdx.x; idx < seq * (D / V); idx += blockDim.x) {
-        const int key = idx / (D / V);
-        const int j0 = (idx - key * (D / V)) * V;
-        Vec<T, V> x = load_vec<T, V>(v_head + (size_t) key * ld + j0);
+    for (int idx = threadIdx.x; idx < (seq / V) * D; idx += blockDim.x) {
+        const int j = idx % D, kg = idx / D;
+        Vec<T, V> x;
 #pragma unroll
-        for (int i = 0; i < V; ++i) vt[(j0 + i) * pitch + key] = x.v[i];
+        for (int i = 0; i < V; ++i) x.v[i] = v_head[(size_t) (kg * V + i) * ld + j];
+        store_vec<T, V>(vt + j * pitch + kg * V, x);
     }
     __syncthreads();
 
@@ -129,19 +234,27 @@ __global__ __launch_bounds__(kBlock) void attention_context_kernel(const T *__re
     const int q_tiles = seq / 32;
     int qt_end = (blockIdx.x + 1) * q_tiles_per_block;
     if (qt_end > q_tiles) qt_end = q_tiles;
-    const int half_k = seq / 2;
+    const int steps = seq / (2 * V);  // reduction slot s of step t in lane half hh is key t*2V + hh*V + s
     for (int qt = blockIdx.x * q_tiles_per_block + wave_in_block(); qt < qt_end; qt += waves) {
-        const T *p_row = probs + ((size_t) bh * seq + qt * 32 + r) * seq + hh * half_k;
+        const T *p_row = probs + ((size_t) bh * seq + qt * 32 + r) * seq + hh * V;
         v16f32 acc[kColTiles];
 #pragma unroll
         for (int jt = 0; jt < kColTiles; ++jt) acc[jt] = v16f32{};
-#pragma unroll 4
-        for (int t = 0; t < half_k / V; ++t) {
-            Vec<T, V> a = load_vec<T, V>(p_row + t * V);
+        for (int t0 = 0; t0 < steps; t0 += kPrefetch) {
+            Vec<T, V> a[kPrefetch];
 #pragma unroll
-            for (int jt = 0; jt < kColTiles; ++jt) {
-                Vec<T, V> bv = *reinterpret_cast<const Vec<T, V> *>(vt + (jt * 32 + r) * pitch + hh * half_k + t * V);
-                Mma<T>::run(acc[jt], a, bv);
+            for (int u = 0; u < kPrefetch; ++u) {
+                a[u] = Vec<T, V>{};
+                if (t0 + u < steps) a[u] = load_vec<T, V>(p_row + (t0 + u) * 2 * V);
+            }
+#pragma unroll
+            for (int u = 0; u < kPrefetch; ++u) {
+                if (t0 + u < steps) {
+#pragma unroll
+                    for (int jt = 0; jt < kColTiles; ++jt) {
+                        Mma<T>::run(acc[jt], a[u], load_vec<T, V>(vt + (jt * 32 + r) * pitch + (t0 + u) * 2 * V + hh * V));
+                    }
+                }
             }
         }
         // lane holds output column jt*32 + r and 16 query rows
@@ -169,6 +282,12 @@ bool shapes_ok(int batch, int heads, int seq, int head_size, int ld, std::initia
 template <typename T, int D>
 int launch_scores(const T *q, const T *k, int ld, T *scores, float alpha, int batch, int heads, int seq,
                   hipStream_t s) {
+    if constexpr (D * sizeof(T) <= 128) {  // a head row is at most one cache line: both operand tiles fit 64 KB of LDS
+        if (seq >= 128) {
+            dim3 grid((seq + 127) / 128, (seq + 127) / 128, batch * heads), block(kBlock);
+            return launch(attention_scores_tiled_kernel<T, D>, grid, block, s, q, k, ld, scores, alpha, seq, heads);
+        }
+    }
     const int key_tiles = seq / 32;
     // keys per wavefront: up to 4 tiles (128 keys) while the grid still has enough workgroups
     const int nt = key_tiles % 4 == 0 && key_tiles >= 16 ? 4 : (key_tiles % 2 == 0 && key_tiles >= 8 ? 2 : 1);
@@ -199,7 +318,8 @@ int launch_context(const T *probs, const T *v, int ld, T *ctx, int ld_ctx, int b
                    hipStream_t s) {
     const int q_tiles = seq / 32;
     const int waves = q_tiles >= 4 ? 4 : q_tiles;
-    const int per_block = waves;  // one query tile per wavefront
+    // query tiles per workgroup: more of them amortise the V^T staging, fewer give more workgroups
+    const int per_block = q_tiles >= 16 ? 8 : waves;
     const size_t lds = (size_t) D * (seq + 16 / sizeof(T)) * sizeof(T);
     if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
     auto kernel = attention_context_kernel<T, D>;
@@ -224,7 +344,6 @@ int attention_context(const T *probs, const T *v, int ld, T *ctx, int ld_ctx, in
     if (!probs || !v || !ctx || batch < 0) return CUBERT_BAD_ARGUMENT;
     if (batch == 0) return 0;
     if (!shapes_ok<T>(batch, heads, seq, head_size, ld, {probs, v}) || ld_ctx < heads * head_size) return CUBERT_UNSUPPORTED;
-    if (seq % (2 * Mma<T>::kVec) != 0) return CUBERT_UNSUPPORTED;
     hipStream_t s = (hipStream_t) stream;
     switch (head_size) {
         case 32: return launch_context<T, 32>(probs, v, ld, ctx, ld_ctx, batch, heads, seq, s);

@@ -309,7 +309,9 @@ def test_gather(K, name, idt):
 
 @pytest.mark.parametrize("name", ["f32", "f16"])
 @pytest.mark.parametrize("batch,heads,seq,d", [(3, 12, 32, 64), (2, 4, 128, 64), (1, 2, 512, 64), (2, 3, 64, 32),
-                                               (1, 2, 96, 128), (2, 16, 128, 64), (5, 1, 32, 64), (1, 2, 256, 64)])
+                                               (1, 2, 96, 128), (2, 16, 128, 64), (5, 1, 32, 64), (1, 2, 256, 64),
+                                               # partial 128 x 128 tiles of the LDS-tiled scores kernel
+                                               (1, 2, 160, 64), (1, 3, 384, 64), (2, 2, 224, 32), (1, 1, 128, 128)])
 def test_attention_scores_and_context(K, name, batch, heads, seq, d):
     rng = np.random.default_rng(batch * 1000 + heads * 100 + seq + d)
     H = heads * d
