@@ -1,0 +1,149 @@
+// Dense layer for a handful of tokens:  C[M, N] = alpha * A[M, K] * B[K, N] + bias  (column-major, no
+// transposes) with N <= 32.  In the row-major picture of a Dense layer A is the weight matrix [in, out]
+// (M = out features, K = in features), B the activations of N tokens and C their outputs.
+//
+// With so few tokens the GEMM is a single pass over the weights: every weight is used once per token and
+// the work is bounded by how fast the weight matrix streams in, i.e. by how much of it is requested at
+// once.  A library GEMM tiled for large N keeps few loads in flight here (a BERT-base forward pass at
+// batch 1, seq 32 spends most of its time in such GEMMs at a few percent of the memory bandwidth).
+//
+// Decomposition: a workgroup of 16 wavefronts owns 32 output features and a slice of K (256 values per
+// pass); each wavefront multiplies a [32 tokens x 16] block of B with a [16 x 32 features] block of A on
+// the matrix cores (v_mfma_f32_32x32x2_f32; fp16 storage is widened to fp32 in registers).  Every load of
+// the wavefront is issued before the first MFMA.  The 16 partial tiles are summed through LDS in wavefront
+// order.  When K is cut into several slices (grid.y > 1) each workgroup stores its partial tile to a
+// workspace and the last workgroup to arrive for a feature block (ticket from an atomic counter) adds the
+// slices in slice order, so the result does not depend on scheduling.
+
+#include "cubert_kernels.h"
+#include "device_common.h"
+
+namespace cubert {
+namespace {
+
+typedef float v16f32 __attribute__((ext_vector_type(16)));
+
+constexpr int kSkinnyWaves = 16;
+constexpr int kSkinnyThreads = kSkinnyWaves * kWave;
+constexpr int kSkinnyChunk = 16;  // reduction values a wavefront consumes per pass: 8 per lane half
+
+// Accumulator register i of the lane half hh holds this row of a 32x32 MFMA result (column = lane % 32).
+__device__ __forceinline__ int acc_row(int i, int hh) { return (i >> 2) * 8 + hh * 4 + (i & 3); }
+
+template <typename T>
+__global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__restrict__ A, int lda,
+                                                                     const T *__restrict__ B, int ldb,
+                                                                     const T *__restrict__ bias, T *__restrict__ C,
+                                                                     int ldc, int M, int N, int K, float alpha,
+                                                                     float *partials, int *counters,
+                                                                     int chunks_per_slice) {
+    __shared__ float red[kSkinnyWaves][32 * 32];
+    constexpr int V = 16 / sizeof(T);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int r = lane & 31, hh = lane >> 5, wave = wave_in_block();
+    const int m0 = blockIdx.x * 32;
+    const int feature = m0 + r;
+    const int chunks = K / kSkinnyChunk;
+    const int c_begin = blockIdx.y * chunks_per_slice;
+    const int c_end = c_begin + chunks_per_slice < chunks ? c_begin + chunks_per_slice : chunks;
+
+    v16f32 acc = v16f32{};
+    for (int c = c_begin + wave; c < c_end; c += kSkinnyWaves) {
+        // reduction slot of MFMA t in lane half hh is k = c*16 + hh*8 + t: the token operand of a lane is 8
+        // consecutive values of one row of B (vector loads), the weight operand one column of 8 rows of A
+        const int kb = c * kSkinnyChunk + hh * 8;
+        float x[8], w[8];
+#pragma unroll
+        for (int u = 0; u < 8 / V; ++u) {
+            Vec<T, V> xv = Vec<T, V>{};
+            if (r < N) xv = load_vec<T, V>(B + (size_t) r * ldb + kb + u * V);
+#pragma unroll
+            for (int e = 0; e < V; ++e) x[u * V + e] = to_f32(xv.v[e]);
+        }
+#pragma unroll
+        for (int t = 0; t < 8; ++t) w[t] = feature < M ? to_f32(A[(size_t) (kb + t) * lda + feature]) : 0.f;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[t], w[t], acc, 0, 0, 0);
+    }
+    // lane holds C[feature = m0 + r, token = acc_row(i, hh)]
+#pragma unroll
+    for (int i = 0; i < 16; ++i) red[wave][acc_row(i, hh) * 32 + r] = acc[i];
+    __syncthreads();
+
+    const int token = threadIdx.x >> 5, f = threadIdx.x & 31;  // one output element per thread
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kSkinnyWaves; ++w) sum += red[w][threadIdx.x];
+    const bool live = token < N && m0 + f < M;
+    const int slices = gridDim.y;
+    if (slices > 1) {
+        // The L2 caches of the chip's dies are not coherent with each other, and a device-scope fence would
+        // write back / invalidate a whole L2 per call.  Instead every access that crosses workgroups is a
+        // relaxed device-scope atomic: such stores write through, such loads read past the die-local cache,
+        // and a store has reached the coherent level once the wavefront's store counter has drained.
+        const size_t pitch = (size_t) gridDim.x * 32;  // features, padded to whole blocks
+        __hip_atomic_store(&partials[((size_t) blockIdx.y * 32 + token) * pitch + m0 + f], sum, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's partial sums are written
+        __syncthreads();                     // ... and so are the other wavefronts' (and red[] is free)
+        int *ticket = reinterpret_cast<int *>(&red[0][0]);
+        if (threadIdx.x == 0) {
+            *ticket = __hip_atomic_fetch_add(&counters[blockIdx.x], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (*ticket != slices - 1) return;
+        // last workgroup of this feature block: every slice's partial tile is complete
+        sum = 0.f;
+        for (int s0 = 0; s0 < slices; s0 += 4) {  // four loads in flight, added in slice order
+            float p[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                p[u] = s0 + u < slices ? __hip_atomic_load(&partials[((size_t) (s0 + u) * 32 + token) * pitch + m0 + f],
+                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                       : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) sum += p[u];
+        }
+        if (threadIdx.x == 0) {  // ready for the next launch
+            __hip_atomic_store(&counters[blockIdx.x], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    if (live) {
+        float v = alpha * sum;
+        if (bias != nullptr) v += to_f32(bias[m0 + f]);
+        C[(size_t) token * ldc + m0 + f] = from_f32<T>(v);
+    }
+}
+
+}  // namespace
+
+// Launches the kernel when the problem fits it, else returns CUBERT_UNSUPPORTED and launches nothing.
+// `partials` holds partial_floats floats, `counters` n_counters ints that are zero between launches.
+template <typename T>
+int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, const T *B, int ldb, T *C, int ldc,
+                const T *bias, float *partials, size_t partial_floats, int *counters, int n_counters,
+                hipStream_t stream) {
+    if (M <= 0 || N <= 0 || N > 32 || K <= 0 || K % kSkinnyChunk != 0) return CUBERT_UNSUPPORTED;
+    if (lda < M || ldb < K || ldc < M) return CUBERT_BAD_ARGUMENT;
+    if (!is_aligned(B, 16) || (ldb * sizeof(T)) % 16 != 0) return CUBERT_UNSUPPORTED;
+    const int blocks = (M + 31) / 32;
+    const int chunks = K / kSkinnyChunk;
+    // one pass per wavefront unless that would need more slices than the workspace holds
+    int chunks_per_slice = kSkinnyWaves;
+    int slices = (chunks + chunks_per_slice - 1) / chunks_per_slice;
+    while (slices > 1 && (size_t) slices * 32 * blocks * 32 > partial_floats) {
+        chunks_per_slice += kSkinnyWaves;
+        slices = (chunks + chunks_per_slice - 1) / chunks_per_slice;
+    }
+    if (blocks > 65535 || slices > 65535 || (slices > 1 && blocks > n_counters)) return CUBERT_UNSUPPORTED;
+    return launch(gemm_skinny_kernel<T>, dim3(blocks, slices), dim3(kSkinnyThreads), stream, A, lda, B, ldb, bias, C,
+                  ldc, M, N, K, alpha, partials, counters, chunks_per_slice);
+}
+
+template int gemm_skinny<float>(int, int, int, float, const float *, int, const float *, int, float *, int,
+                                const float *, float *, size_t, int *, int, hipStream_t);
+template int gemm_skinny<half_t>(int, int, int, float, const half_t *, int, const half_t *, int, half_t *, int,
+                                 const half_t *, float *, size_t, int *, int, hipStream_t);
+
+}  // namespace cubert

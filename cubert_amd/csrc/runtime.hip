@@ -22,6 +22,12 @@
 #include "device_common.h"
 
 namespace cubert {
+// kernels/gemm_skinny.hip
+template <typename T>
+int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, const T *B, int ldb, T *C, int ldc,
+                const T *bias, float *partials, size_t partial_floats, int *counters, int n_counters,
+                hipStream_t stream);
+
 LaunchTiming &pending_launch_timing() {
     static thread_local LaunchTiming pending;
     return pending;
@@ -43,6 +49,9 @@ hipMemcpyKind copy_kind(int kind) {
 }
 
 constexpr size_t kWorkspaceBytes = 64u << 20;
+// scratch of the few-token GEMM kernel: partial tiles (fp32) and one arrival counter per feature block
+constexpr size_t kSkinnyPartialFloats = 1u << 20;
+constexpr int kSkinnyCounters = 4096;
 
 struct GemmKey {
     int type;  // 0 = f32, 1 = f16
@@ -69,6 +78,8 @@ struct BlasContext {
     hipblasLtHandle_t lt = nullptr;
     hipStream_t stream = nullptr;
     void *workspace = nullptr;
+    float *skinny_partials = nullptr;
+    int *skinny_counters = nullptr;  // zero between launches (the kernel resets what it counted)
     std::map<GemmKey, GemmPlan> plans;
     std::mutex mutex;
 };
@@ -184,12 +195,34 @@ int run_naive_gemm(hipStream_t stream, int type, int transA, int transB, int M, 
     return hip_rc(hipGetLastError());
 }
 
+bool gemm_mode_is(const char *mode) {
+    const char *v = getenv("CUBERT_GEMM");
+    return v != nullptr && std::string(v) == mode;
+}
+
 bool force_naive_gemm() {
-    static const bool forced = [] {
-        const char *v = getenv("CUBERT_GEMM");
-        return v != nullptr && std::string(v) == "naive";
-    }();
+    static const bool forced = gemm_mode_is("naive");
     return forced;
+}
+
+// CUBERT_GEMM=library sends every GEMM to hipBLASLt, also those the few-token kernel would take.
+bool library_gemm_only() {
+    static const bool forced = gemm_mode_is("library");
+    return forced;
+}
+
+int run_skinny(BlasContext *ctx, int type, int M, int N, int K, float alpha, const void *A, int lda, const void *B,
+               int ldb, void *C, int ldc, const void *bias) {
+    if (type == 0) {
+        return cubert::gemm_skinny<float>(M, N, K, alpha, (const float *) A, lda, (const float *) B, ldb, (float *) C,
+                                          ldc, (const float *) bias, ctx->skinny_partials, kSkinnyPartialFloats,
+                                          ctx->skinny_counters, kSkinnyCounters, ctx->stream);
+    }
+    return cubert::gemm_skinny<cubert::half_t>(M, N, K, alpha, (const cubert::half_t *) A, lda,
+                                               (const cubert::half_t *) B, ldb, (cubert::half_t *) C, ldc,
+                                               (const cubert::half_t *) bias, ctx->skinny_partials,
+                                               kSkinnyPartialFloats, ctx->skinny_counters, kSkinnyCounters,
+                                               ctx->stream);
 }
 
 int run_gemm(void *handle, int type, int transA, int transB, int M, int N, int K, float alpha, const void *A, int lda,
@@ -203,6 +236,10 @@ int run_gemm(void *handle, int type, int transA, int transB, int M, int N, int K
     if (force_naive_gemm()) {
         return run_naive_gemm(ctx->stream, type, transA, transB, M, N, K, alpha, A, lda, strideA, B, ldb, strideB,
                               beta, C, ldc, strideC, batch, bias);
+    }
+    if (!transA && !transB && batch == 1 && beta == 0.f && N <= 32 && !library_gemm_only()) {
+        const int rc = run_skinny(ctx, type, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias);
+        if (rc != CUBERT_UNSUPPORTED) return rc;
     }
     std::lock_guard<std::mutex> lock(ctx->mutex);
     auto it = ctx->plans.find(key);
@@ -314,7 +351,13 @@ void *cubert_blas_create(void) {
         delete ctx;
         return nullptr;
     }
-    if (hipMalloc(&ctx->workspace, kWorkspaceBytes) != hipSuccess) {
+    if (hipMalloc(&ctx->workspace, kWorkspaceBytes) != hipSuccess ||
+        hipMalloc((void **) &ctx->skinny_partials, kSkinnyPartialFloats * sizeof(float)) != hipSuccess ||
+        hipMalloc((void **) &ctx->skinny_counters, kSkinnyCounters * sizeof(int)) != hipSuccess ||
+        hipMemset(ctx->skinny_counters, 0, kSkinnyCounters * sizeof(int)) != hipSuccess) {
+        (void) hipFree(ctx->workspace);
+        (void) hipFree(ctx->skinny_partials);
+        (void) hipFree(ctx->skinny_counters);
         hipblasLtDestroy(ctx->lt);
         delete ctx;
         return nullptr;
@@ -333,6 +376,8 @@ int cubert_blas_destroy(void *handle) {
         if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
     }
     (void) hipFree(ctx->workspace);
+    (void) hipFree(ctx->skinny_partials);
+    (void) hipFree(ctx->skinny_counters);
     hipblasLtDestroy(ctx->lt);
     delete ctx;
     return 0;
@@ -355,6 +400,20 @@ int cubert_gemm_f16(void *handle, int transA, int transB, int M, int N, int K, f
                     int lda, const cubert_half *B, int ldb, float beta, cubert_half *C, int ldc,
                     const cubert_half *bias) {
     return run_gemm(handle, 1, transA, transB, M, N, K, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc, 0, 1, bias);
+}
+
+int cubert_gemm_skinny_f32(void *handle, int M, int N, int K, float alpha, const float *A, int lda, const float *B,
+                           int ldb, float *C, int ldc, const float *bias) {
+    BlasContext *ctx = (BlasContext *) handle;
+    if (!ctx || !A || !B || !C) return CUBERT_BAD_ARGUMENT;
+    return run_skinny(ctx, 0, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias);
+}
+
+int cubert_gemm_skinny_f16(void *handle, int M, int N, int K, float alpha, const cubert_half *A, int lda,
+                           const cubert_half *B, int ldb, cubert_half *C, int ldc, const cubert_half *bias) {
+    BlasContext *ctx = (BlasContext *) handle;
+    if (!ctx || !A || !B || !C) return CUBERT_BAD_ARGUMENT;
+    return run_skinny(ctx, 1, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias);
 }
 
 int cubert_gemm_strided_batch_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha,

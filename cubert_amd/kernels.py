@@ -144,6 +144,15 @@ class Blas(object):
               ldb, float(beta), _ptr(C), ldc, _ptr(bias))
         return C
 
+    def gemm_skinny(self, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias=None):
+        """C = alpha A B (+ bias) with the few-token kernel (N <= 32); None when the problem does not fit it."""
+        fn = getattr(lib(), "cubert_gemm_skinny_" + _suffix(C))
+        rc = fn(self.handle, M, N, K, float(alpha), _ptr(A), lda, _ptr(B), ldb, _ptr(C), ldc, _ptr(bias))
+        if rc == -2:
+            return None
+        _check(rc, fn.__name__)
+        return C
+
     def gemm_strided_batch(self, transA, transB, M, N, K, alpha, A, lda, sA, B, ldb, sB, beta, C, ldc, sC, batch):
         _call("cubert_gemm_strided_batch", C, self.handle, int(transA), int(transB), M, N, K, float(alpha), _ptr(A),
               lda, sA, _ptr(B), ldb, sB, float(beta), _ptr(C), ldc, sC, batch)

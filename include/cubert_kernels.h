@@ -170,6 +170,20 @@ int cubert_gemm_f16(void *handle, int transA, int transB, int M, int N, int K, f
                     const cubert_half *A, int lda, const cubert_half *B, int ldb, float beta, cubert_half *C,
                     int ldc, const cubert_half *bias);
 
+/* C = alpha * A * B + bias for N <= 32 columns (no transposes, beta = 0): the Dense layer of a request with at
+ * most 32 tokens, where A is the [in, out] weight matrix (M = out, K = in) and each column of B one token.
+ * One pass over the weights on the matrix cores with every load in flight at once; K is cut into slices that
+ * are added in a fixed order, so results do not depend on scheduling.  cubert_gemm_* takes this path by
+ * itself when the problem fits (CUBERT_GEMM=library in the environment turns that off).  Needs K a multiple
+ * of 16 and B 16-byte aligned with ldb a multiple of 16 bytes; anything else returns CUBERT_UNSUPPORTED and
+ * launches nothing.  Calls on one handle must not overlap (they share the handle's scratch).
+ * replaces: Dense<T>::compute -> blas_gemm<T> for small batch * seq_length, reference
+ * src/cuBERT/op/Dense.cpp:47-57 (bias: Dense.cpp:41-44). */
+int cubert_gemm_skinny_f32(void *handle, int M, int N, int K, float alpha, const float *A, int lda, const float *B,
+                           int ldb, float *C, int ldc, const float *bias);
+int cubert_gemm_skinny_f16(void *handle, int M, int N, int K, float alpha, const cubert_half *A, int lda,
+                           const cubert_half *B, int ldb, cubert_half *C, int ldc, const cubert_half *bias);
+
 /* The same over `batch_count` problems at fixed strides (in elements).
  * replaces: blas_gemm_strided_batch<T>, reference src/cuBERT/common.h:82-92. */
 int cubert_gemm_strided_batch_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha,

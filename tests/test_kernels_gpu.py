@@ -369,6 +369,55 @@ def test_gemm_against_oracle_sgemm(K, name, ta, tb, M, N, K_):
         assert_close(host(C), want, 2e-5 if name == "f32" else 2e-3, "gemm %s beta=%g bias=%s" % (name, beta, use_bias))
 
 
+# ------------------------------------------------------------------ few-token Dense GEMM
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("M,N,K_", [(768, 32, 768), (2304, 32, 768), (3072, 32, 768), (768, 32, 3072), (768, 1, 768),
+                                    (100, 7, 64), (33, 32, 16), (1024, 16, 4096), (2, 5, 768), (768, 32, 272)])
+def test_gemm_skinny_against_oracle_sgemm(K, name, M, N, K_):
+    """Dense layer of a request with at most 32 tokens (column-major C[M,N] = A[M,K] B[K,N] + bias), K cut into
+    1..16 slices; 30 launches in a row must give bit-identical results (slices are added in a fixed order and
+    the arrival counters reset themselves)."""
+    rng = np.random.default_rng(M + N + K_)
+    ldb = K_ + 8  # a padded activation row pitch (multiple of 16 bytes), as a strided first-token view has
+    A = q(rng.normal(0, 1, M * K_), name)
+    Bs = [q(rng.normal(0, 1, N * ldb), name) for _ in range(2)]  # alternate: stale partial sums would show
+    bias = q(rng.normal(0, 1, M), name)
+    blas = K.Blas()
+    dA, dBs, dbias = dev(A, tdt(name)), [dev(B, tdt(name)) for B in Bs], dev(bias, tdt(name))
+    for alpha, use_bias in ((1.0, True), (0.5, False)):
+        outs = [[], []]
+        for it in range(30):
+            C = torch.full((N * M,), 7.0, dtype=tdt(name), device="cuda")
+            assert blas.gemm_skinny(M, N, K_, alpha, dA, M, dBs[it % 2], ldb, C, M,
+                                    bias=dbias if use_bias else None) is not None
+            outs[it % 2].append(C)
+        for which in range(2):
+            for other in outs[which][1:]:
+                assert torch.equal(outs[which][0], other)
+            want = oracle.sgemm(0, 0, M, N, K_, alpha, A, M, Bs[which], ldb, 0.0, np.zeros(N * M, np.float32), M)
+            if use_bias:
+                want = (want.reshape(N, M) + bias[None, :]).ravel()
+            assert_close(host(outs[which][0]), want, 2e-5 if name == "f32" else 2e-3,
+                         "gemm_skinny %s alpha=%g" % (name, alpha))
+    B, dB = Bs[0], dBs[0]
+    # the general entry point takes the same path by itself
+    C = torch.zeros((N * M,), dtype=tdt(name), device="cuda")
+    blas.gemm(0, 0, M, N, K_, 1.0, dA, M, dB, ldb, 0.0, C, M, bias=dbias)
+    want = (oracle.sgemm(0, 0, M, N, K_, 1.0, A, M, B, ldb, 0.0, np.zeros(N * M, np.float32), M).reshape(N, M)
+            + bias[None, :]).ravel()
+    assert_close(host(C), want, 2e-5 if name == "f32" else 2e-3, "gemm via skinny %s" % name)
+
+
+def test_gemm_skinny_declines_what_it_cannot_do(K):
+    blas = K.Blas()
+    x = torch.zeros(64 * 1024, device="cuda")
+    assert blas.gemm_skinny(64, 33, 64, 1.0, x, 64, x, 64, x, 64) is None      # more than 32 tokens
+    assert blas.gemm_skinny(64, 8, 24, 1.0, x, 64, x, 24, x, 64) is None       # K not a multiple of 16
+    assert blas.gemm_skinny(64, 8, 32, 1.0, x, 64, x[1:], 32, x, 64) is None   # misaligned activations
+    assert blas.gemm_skinny(64, 8, 32, 1.0, x, 64, x, 34, x, 64) is None       # row pitch not 16-byte aligned
+
+
 # ------------------------------------------------------------------ edge cases
 
 def test_empty_and_bad_arguments(K):
