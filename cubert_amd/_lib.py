@@ -85,6 +85,7 @@ for _t in ("f32", "f16"):
         "cubert_mask_scale_softmax_" + _t: (ci, [vp, vp, cf, ci, ci, ci, vp]),
         "cubert_row_softmax_" + _t: (ci, [vp, vp, ci, ci, vp]),
         "cubert_attention_scores_" + _t: (ci, [vp, vp, ci, vp, cf, ci, ci, ci, ci, vp]),
+        "cubert_attention_fused_" + _t: (ci, [vp, vp, vp, ci, vp, vp, ci, cf, ci, ci, ci, ci, vp]),
         "cubert_attention_context_" + _t: (ci, [vp, vp, ci, vp, ci, ci, ci, ci, ci, vp]),
         "cubert_bias_tanh_" + _t: (ci, [vp, vp, ci, ci, vp]),
         "cubert_mean_pool_" + _t: (ci, [vp, vp, ci, ci, ci, vp]),

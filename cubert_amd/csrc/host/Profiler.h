@@ -24,7 +24,8 @@ public:
         kRowSoftmax = 6,
         kDenseGemm = 7,
         kAttentionGemm = 8,
-        kKinds = 9
+        kAttentionFused = 9,
+        kKinds = 10
     };
 
     ~Profiler() {
@@ -42,10 +43,10 @@ public:
 
     bool on(Kind k) const { return (mask >> k) & 1u; }
 
-    // The layer kernels (kinds 0..6) are one launch each: the launch itself carries the event pair and
-    // the elapsed time is the kernel's execution time.  GEMM kinds may be several library launches, so
-    // they are bracketed by marker events (which adds the gaps between launches).
-    static bool single_launch(Kind k) { return k < kDenseGemm; }
+    // The layer kernels (kinds 0..6) and the fused attention kernel are one launch each: the launch itself
+    // carries the event pair and the elapsed time is the kernel's execution time.  GEMM kinds may be several
+    // library launches, so they are bracketed by marker events (which adds the gaps between launches).
+    static bool single_launch(Kind k) { return k < kDenseGemm || k == kAttentionFused; }
 
     void begin(Kind k, void *stream) {
         if (!on(k)) return;

@@ -1,6 +1,8 @@
 #include "Transformer.h"
 
 #include <cmath>
+#include <cstdlib>
+#include <string>
 #include <stdexcept>
 
 namespace cuBERT {
@@ -120,6 +122,17 @@ void Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *ma
     const T *Q = qkv, *K = qkv + H, *V = qkv + 2 * H;
     const long long seq_stride = (long long) S * ld, head_stride = d;
     const long long score_b = (long long) A * S * S, score_a = (long long) S * S;
+
+    // Short sequences: one launch, the score tensor stays in registers.  CUBERT_ATTENTION=split in the
+    // environment keeps the three-operator path below (scores, mask + softmax, context) for every shape.
+    static const bool split_only = [] {
+        const char *e = std::getenv("CUBERT_ATTENTION");
+        return e != nullptr && std::string(e) == "split";
+    }();
+    if (!split_only) {
+        Timed t(profiler, Profiler::kAttentionFused, stream);
+        if (cuBERT::attention_fused(Q, K, V, ld, mask, context_out, H, alpha, B, A, S, d, stream)) return;
+    }
 
     const bool loop_heads = A <= B;
     const int outer = loop_heads ? A : B, inner = loop_heads ? B : A;

@@ -185,6 +185,25 @@ inline bool attention_context(const half *probs, const half *v, int ld, half *ct
     return true;
 }
 
+// The whole attention core (scores, mask, softmax, context) in one launch for seq_length <= 128; false when
+// the shape has no such kernel (reference: AttentionSelf.cpp:96-111 runs it as three operators).
+inline bool attention_fused(const float *q, const float *k, const float *v, int ld, const int8_t *mask, float *ctx,
+                            int ld_ctx, float alpha, int batch, int heads, int seq, int head_size, void *stream) {
+    const int rc = cubert_attention_fused_f32(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, head_size,
+                                              stream);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+inline bool attention_fused(const half *q, const half *k, const half *v, int ld, const int8_t *mask, half *ctx,
+                            int ld_ctx, float alpha, int batch, int heads, int seq, int head_size, void *stream) {
+    const int rc = cubert_attention_fused_f16(h(q), h(k), h(v), ld, mask, h(ctx), ld_ctx, alpha, batch, heads, seq,
+                                              head_size, stream);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+
 // reference: op/Softmax.h:8-14
 inline void softmax_(const float *in, float *out, int rows, int channel, void *stream) {
     CUBERT_CHECK(cubert_row_softmax_f32(in, out, rows, channel, stream));

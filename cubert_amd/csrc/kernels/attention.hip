@@ -267,6 +267,174 @@ __global__ __launch_bounds__(kBlock) void attention_context_kernel(const T *__re
     }
 }
 
+// ---- whole attention core in one launch for short sequences (seq <= 128) ----
+// ctx = softmax(alpha * Q K^T + mask) V per (batch, head) without the [batch, heads, seq, seq] tensor ever
+// leaving the registers.  A workgroup owns one (batch, head) problem: its seq/32 wavefronts take 32 queries
+// each and share K, V and the mask, staged once in LDS by coalesced loads that are all issued up front.
+// The score tiles are computed transposed (A = key rows, B = query rows), so lane (r, hh) ends up with query
+// r and 16 keys per key tile: the softmax statistics of a query are an in-lane reduction plus one exchange
+// with lane r + 32.  The lane's probabilities are then exactly the A operand slots of the second contraction:
+// a reduction slot may be any key as long as the B operand names the same key, so V is staged transposed
+// ([head column][key]) with the keys permuted into slot order and a lane's B operand is one 16-byte LDS read.
+// P never moves.  Scores and probabilities are rounded to the storage type at the points where the
+// three-kernel path stores them, which keeps the two paths within summation-order differences of each other.
+constexpr float kMaskedScore = -10000.0f;
+
+template <typename T>
+__device__ __forceinline__ float normalise_prob(float e, float sum, float inv_sum);
+template <>
+__device__ __forceinline__ float normalise_prob<float>(float e, float sum, float) { return e / sum; }
+template <>
+__device__ __forceinline__ float normalise_prob<half_t>(float e, float, float inv_sum) { return e * inv_sum; }
+
+// LDS bytes of attention_fused_kernel<T, D, KT>: K rows, V^T rows (both padded by 16 bytes), additive mask.
+template <typename T, int D, int KT>
+constexpr size_t fused_lds_bytes() {
+    constexpr int V = 16 / sizeof(T), S = KT * 32;
+    return (size_t) S * (D + V) * sizeof(T) + (size_t) D * (S + V) * sizeof(T) + S * sizeof(float);
+}
+
+// grid = batch * heads workgroups of KT wavefronts; seq = 32 * KT.
+template <typename T, int D, int KT>
+__global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__restrict__ q, const T *__restrict__ k,
+                                                                     const T *__restrict__ v, int ld,
+                                                                     const int8_t *__restrict__ mask,
+                                                                     T *__restrict__ ctx, int ld_ctx, float alpha,
+                                                                     int heads) {
+    constexpr int V = Mma<T>::kVec;
+    constexpr int kSteps = D / 2 / V;
+    constexpr int kColTiles = D / 32;
+    constexpr int S = KT * 32;
+    constexpr int kThreads = KT * kWave;
+    constexpr int kPitchK = D + V;  // +16 bytes: conflict-free 16-byte reads down a column of rows
+    constexpr int kPitchV = S + V;
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *s_k = reinterpret_cast<T *>(smem);                 // [S][kPitchK]
+    T *s_vt = s_k + S * kPitchK;                          // [D][kPitchV], keys in slot order
+    float *s_mask = reinterpret_cast<float *>(s_vt + D * kPitchV);  // [S] additive mask
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int r = lane & 31, hh = lane >> 5;
+    const int qt = wave_in_block();
+    const int bh = blockIdx.x;
+    const int b = bh / heads, h = bh - b * heads;
+    const T *k_head = k + (size_t) b * S * ld + (size_t) h * D;
+    const T *v_head = v + (size_t) b * S * ld + (size_t) h * D;
+
+    // this wavefront's query operand, straight from memory: lane half hh takes head columns hh*D/2 .. +D/2
+    const T *q_row = q + ((size_t) b * S + qt * 32 + r) * ld + (size_t) h * D + hh * (D / 2);
+    Vec<T, V> qv[kSteps];
+#pragma unroll
+    for (int t = 0; t < kSteps; ++t) qv[t] = load_vec<T, V>(q_row + t * V);
+
+    // K: S rows of D/V vectors.  V^T: for head column j and slot group (kt, u, half) the V keys
+    // kt*32 + acc_row(u*V + e, half), e < V, go to positions kt*32 + u*2V + half*V + e of row j.
+    constexpr int kVecPerRow = D / V;
+    constexpr int kLoadsK = S * kVecPerRow / kThreads;    // = D / V / 2
+    constexpr int kGroups = S / V;                        // slot groups per head column
+    constexpr int kLoadsV = kGroups * D / kThreads;       // = D / V / 2
+    Vec<T, V> kreg[kLoadsK], vreg[kLoadsV];
+#pragma unroll
+    for (int u = 0; u < kLoadsK; ++u) {
+        const int idx = threadIdx.x + u * kThreads;
+        const int row = idx / kVecPerRow, c = idx - row * kVecPerRow;
+        kreg[u] = load_vec<T, V>(k_head + (size_t) row * ld + c * V);
+    }
+#pragma unroll
+    for (int u = 0; u < kLoadsV; ++u) {
+        const int idx = threadIdx.x + u * kThreads;
+        const int j = idx % D, grp = idx / D;             // consecutive threads: consecutive columns (coalesced)
+        const int kt = grp / (32 / V), in_tile = grp % (32 / V);
+        const int run = in_tile >> 1, half = in_tile & 1;
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+            vreg[u].v[e] = v_head[(size_t) (kt * 32 + acc_row(run * V + e, half)) * ld + j];
+        }
+    }
+    for (int i = threadIdx.x; i < S; i += kThreads) {
+        s_mask[i] = (mask != nullptr && !mask[(size_t) b * S + i]) ? kMaskedScore : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < kLoadsK; ++u) {
+        const int idx = threadIdx.x + u * kThreads;
+        const int row = idx / kVecPerRow, c = idx - row * kVecPerRow;
+        store_vec<T, V>(s_k + row * kPitchK + c * V, kreg[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kLoadsV; ++u) {
+        const int idx = threadIdx.x + u * kThreads;
+        const int j = idx % D, grp = idx / D;
+        store_vec<T, V>(s_vt + j * kPitchV + grp * V, vreg[u]);
+    }
+    __syncthreads();
+
+    // scores^T[key, query]
+    v16f32 p[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        v16f32 c = {};
+#pragma unroll
+        for (int t = 0; t < kSteps; ++t) {
+            Mma<T>::run(c, load_vec<T, V>(s_k + (kt * 32 + r) * kPitchK + hh * (D / 2) + t * V), qv[t]);
+        }
+        p[kt] = c;
+    }
+
+    // register i of tile kt: key kt*32 + acc_row(i, hh), query qt*32 + r
+    float mx = -3.402823466e+38f;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const Vec<float, 4> m = load_vec<float, 4>(s_mask + kt * 32 + g * 8 + hh * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float sc = to_f32(from_f32<T>(p[kt][g * 4 + e] * alpha)) + m.v[e];
+                p[kt][g * 4 + e] = sc;
+                mx = fmaxf(mx, sc);
+            }
+        }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    float sum = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            p[kt][i] = __expf(p[kt][i] - mx);
+            sum += p[kt][i];
+        }
+    }
+    sum += __shfl_xor(sum, 32, kWave);
+    const float inv = 1.f / sum;
+
+    // ctx[query, column]: A slots = this lane's probabilities, B = the same keys of V^T row (column) jt*32 + r
+    v16f32 out[kColTiles];
+#pragma unroll
+    for (int jt = 0; jt < kColTiles; ++jt) out[jt] = v16f32{};
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+        for (int run = 0; run < 16 / V; ++run) {
+            Vec<T, V> a;
+#pragma unroll
+            for (int e = 0; e < V; ++e) a.v[e] = from_f32<T>(normalise_prob<T>(p[kt][run * V + e], sum, inv));
+#pragma unroll
+            for (int jt = 0; jt < kColTiles; ++jt) {
+                Mma<T>::run(out[jt], a,
+                            load_vec<T, V>(s_vt + (jt * 32 + r) * kPitchV + kt * 32 + run * 2 * V + hh * V));
+            }
+        }
+    }
+    // lane holds output column jt*32 + r and 16 query rows
+    T *dst = ctx + ((size_t) b * S + qt * 32) * ld_ctx + (size_t) h * D + r;
+#pragma unroll
+    for (int jt = 0; jt < kColTiles; ++jt) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dst[(size_t) acc_row(i, hh) * ld_ctx + jt * 32] = from_f32<T>(out[jt][i]);
+    }
+}
+
 template <typename T>
 bool shapes_ok(int batch, int heads, int seq, int head_size, int ld, std::initializer_list<const void *> ptrs) {
     constexpr int V = Mma<T>::kVec;
@@ -352,6 +520,56 @@ int attention_context(const T *probs, const T *v, int ld, T *ctx, int ld_ctx, in
     }
 }
 
+template <typename T, int D, int KT>
+int launch_fused_kt(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
+                    int batch, int heads, hipStream_t s) {
+    constexpr size_t lds = fused_lds_bytes<T, D, KT>();
+    if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
+    auto kernel = attention_fused_kernel<T, D, KT>;
+    if (lds > 48 * 1024) {
+        static thread_local bool raised = false;  // per instantiation and thread; the call is cheap and idempotent
+        if (!raised) {
+            if (hipFuncSetAttribute((const void *) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) !=
+                hipSuccess) {
+                (void) hipGetLastError();
+                return CUBERT_UNSUPPORTED;
+            }
+            raised = true;
+        }
+    }
+    return launch_lds(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask, ctx, ld_ctx,
+                      alpha, heads);
+}
+
+template <typename T, int D>
+int launch_fused(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
+                 int batch, int heads, int seq, hipStream_t s) {
+    switch (seq / 32) {
+        case 1: return launch_fused_kt<T, D, 1>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, s);
+        case 2: return launch_fused_kt<T, D, 2>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, s);
+        case 3: return launch_fused_kt<T, D, 3>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, s);
+        case 4: return launch_fused_kt<T, D, 4>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, s);
+        default: return CUBERT_UNSUPPORTED;
+    }
+}
+
+template <typename T>
+int attention_fused(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
+                    int batch, int heads, int seq, int head_size, void *stream) {
+    if (batch == 0 || heads == 0 || seq == 0) return 0;
+    if (!q || !k || !v || !ctx || batch < 0 || heads < 0 || seq < 0 || head_size <= 0) return CUBERT_BAD_ARGUMENT;
+    if (ld < heads * head_size) return CUBERT_BAD_ARGUMENT;
+    if (seq > 128 || !shapes_ok<T>(batch, heads, seq, head_size, ld, {q, k, v}) || ld_ctx < heads * head_size) {
+        return CUBERT_UNSUPPORTED;
+    }
+    hipStream_t s = (hipStream_t) stream;
+    switch (head_size) {
+        case 32: return launch_fused<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, s);
+        case 64: return launch_fused<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, s);
+        default: return launch_fused<T, 128>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, s);
+    }
+}
+
 }  // namespace
 }  // namespace cubert
 
@@ -376,4 +594,19 @@ extern "C" int cubert_attention_context_f16(const cubert_half *probs, const cube
                                             void *stream) {
     return cubert::attention_context<half_t>((const half_t *) probs, (const half_t *) v, ld, (half_t *) ctx, ld_ctx,
                                              batch, heads, seq_length, head_size, stream);
+}
+
+extern "C" int cubert_attention_fused_f32(const float *q, const float *k, const float *v, int ld, const int8_t *mask,
+                                          float *ctx, int ld_ctx, float alpha, int batch, int heads, int seq_length,
+                                          int head_size, void *stream) {
+    return cubert::attention_fused<float>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq_length, head_size,
+                                          stream);
+}
+
+extern "C" int cubert_attention_fused_f16(const cubert_half *q, const cubert_half *k, const cubert_half *v, int ld,
+                                          const int8_t *mask, cubert_half *ctx, int ld_ctx, float alpha, int batch,
+                                          int heads, int seq_length, int head_size, void *stream) {
+    return cubert::attention_fused<cubert::half_t>((const cubert::half_t *) q, (const cubert::half_t *) k,
+                                                   (const cubert::half_t *) v, ld, mask, (cubert::half_t *) ctx,
+                                                   ld_ctx, alpha, batch, heads, seq_length, head_size, stream);
 }

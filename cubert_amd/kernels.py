@@ -89,6 +89,20 @@ def attention_scores(qkv, batch, heads, seq, head_size, alpha):
     return scores
 
 
+def attention_fused(qkv, mask, batch, heads, seq, head_size, alpha):
+    """ctx[B*S, H] = softmax(alpha Q K^T + mask) V in one launch (seq <= 128); None when the shape does not fit."""
+    hidden = heads * head_size
+    flat = qkv.view(-1)
+    ctx = torch.empty((batch * seq, hidden), dtype=qkv.dtype, device=qkv.device)
+    fn = getattr(lib(), "cubert_attention_fused_" + _suffix(qkv))
+    rc = fn(_ptr(flat), _ptr(flat[hidden:]), _ptr(flat[2 * hidden:]), 3 * hidden, _ptr(mask), _ptr(ctx), hidden,
+            float(alpha), batch, heads, seq, head_size, _stream())
+    if rc == -2:
+        return None
+    _check(rc, fn.__name__)
+    return ctx
+
+
 def attention_context(probs, qkv, batch, heads, seq, head_size):
     """ctx[B*S, H] = P V with V the third column block of the packed projection."""
     hidden = heads * head_size

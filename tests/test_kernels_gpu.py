@@ -335,6 +335,48 @@ def test_attention_scores_and_context(K, name, batch, heads, seq, d):
     assert_close(host(ctx), want_ctx, 2e-5 if name == "f32" else 2e-3, "attention_context %s" % name)
 
 
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("batch,heads,seq,d", [(3, 12, 32, 64), (2, 4, 128, 64), (2, 3, 64, 32), (1, 2, 96, 128),
+                                               (2, 16, 128, 64), (5, 1, 32, 64), (7, 3, 64, 64)])
+@pytest.mark.parametrize("masked", [True, False])
+def test_attention_fused_against_oracle(K, name, batch, heads, seq, d, masked):
+    """One-launch attention core vs the oracle's attention_self pieces (att_q_k -> mask -> softmax -> att_qk_v),
+    with an arbitrary 0/1 mask pattern (not only prefixes) and one fully masked sequence."""
+    rng = np.random.default_rng(batch * 1000 + heads * 100 + seq + d)
+    H = heads * d
+    qkv = q(rng.normal(0, 1, (batch * seq, 3 * H)), name)
+    qh, kh, vh = (np.ascontiguousarray(x) for x in (qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:]))
+    mask = (rng.random((batch, seq)) < 0.7).astype(np.int8)
+    mask[0, :] = 0
+    alpha = 1.0 / math.sqrt(d)
+    ctx = K.attention_fused(dev(qkv, tdt(name)), dev(mask) if masked else None, batch, heads, seq, d, alpha)
+    assert ctx is not None
+    scores = oracle.att_q_k(qh, kh, batch, seq, heads, d, alpha=alpha)  # [B, S_q, A, S_k]
+    if name == "f16":
+        scores = oracle.round_to_half(scores)  # the scaled scores are what is stored; the mask is added in fp32
+    if masked:
+        scores = scores + (-10000.0 * (1.0 - mask.astype(np.float32)))[:, None, None, :]
+    p = oracle.softmax_(np.ascontiguousarray(scores.reshape(-1, seq), dtype=np.float32)).reshape(scores.shape)
+    if name == "f16":
+        p = oracle.round_to_half(p)
+    want = oracle.att_qk_v(np.ascontiguousarray(p, dtype=np.float32), vh, batch, seq, heads, d).reshape(batch * seq, H)
+    # Sequence 0 is fully masked: every score sits at -10000, where fp32 resolves 1e-3, so a last-bit difference
+    # in a score moves its probability by 1e-3 relative.  It gets the fp16 tolerance; the others the tight one.
+    tol = 2e-5 if name == "f32" else 2e-3
+    first = seq if masked else 0
+    if first < batch * seq:
+        assert_close(host(ctx)[first:], want[first:], tol, "attention_fused %s" % name)
+    assert_close(host(ctx)[:seq], want[:seq], 2e-3, "attention_fused %s, fully masked sequence" % name)
+    # and against the three-kernel sequence of this library
+    s3 = K.attention_scores(dev(qkv, tdt(name)), batch, heads, seq, d, alpha)
+    K.mask_scale_softmax_(s3, dev(mask) if masked else None, 1.0)
+    c3 = K.attention_context(s3, dev(qkv, tdt(name)), batch, heads, seq, d)
+    if first < batch * seq:
+        assert_close(host(ctx)[first:], host(c3)[first:], 1e-5 if name == "f32" else 2e-3,
+                     "fused vs three kernels %s" % name)
+    assert_close(host(ctx)[:seq], host(c3)[:seq], 2e-3, "fused vs three kernels %s, fully masked sequence" % name)
+
+
 def test_attention_unsupported_shapes_are_declined(K):
     """Shapes without a matrix-core kernel return CUBERT_UNSUPPORTED and launch nothing; the host classes then
     loop the strided-batched GEMM (covered by the encoder reference vectors, seq 4, head size 3)."""
@@ -343,6 +385,8 @@ def test_attention_unsupported_shapes_are_declined(K):
     assert K.attention_context(torch.zeros((2, 2, 4, 4), device="cuda"), qkv, 2, 2, 4, 3) is None
     qkv = torch.zeros((2 * 40, 3 * 128), device="cuda")
     assert K.attention_scores(qkv, 2, 2, 40, 64, 1.0) is None  # seq not a multiple of 32
+    qkv = torch.zeros((160, 3 * 128), device="cuda")
+    assert K.attention_fused(qkv, None, 1, 2, 160, 64, 1.0) is None   # longer than the fused kernel holds
 
 
 # ------------------------------------------------------------------ GEMM convention
