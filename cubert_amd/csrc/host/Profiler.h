@@ -43,10 +43,11 @@ public:
 
     bool on(Kind k) const { return (mask >> k) & 1u; }
 
-    // The layer kernels (kinds 0..6) and the fused attention kernel are one launch each: the launch itself
-    // carries the event pair and the elapsed time is the kernel's execution time.  GEMM kinds may be several
-    // library launches, so they are bracketed by marker events (which adds the gaps between launches).
-    static bool single_launch(Kind k) { return k < kDenseGemm || k == kAttentionFused; }
+    // The layer kernels (kinds 0..6) are one launch each: the launch itself carries the event pair and
+    // the elapsed time is the kernel's execution time.  GEMM kinds may be several library launches, so
+    // they are bracketed by marker events (which adds the gaps between launches), and so is the fused
+    // attention kernel.
+    static bool single_launch(Kind k) { return k < kDenseGemm; }
 
     void begin(Kind k, void *stream) {
         if (!on(k)) return;

@@ -123,15 +123,17 @@ void Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *ma
     const long long seq_stride = (long long) S * ld, head_stride = d;
     const long long score_b = (long long) A * S * S, score_a = (long long) S * S;
 
-    // Short sequences: one launch, the score tensor stays in registers.  CUBERT_ATTENTION=split in the
+    // One launch with the score tensor held in registers where the shape allows (seq_length <= 512, K and V
+    // of a head within LDS).  CUBERT_ATTENTION=split in the
     // environment keeps the three-operator path below (scores, mask + softmax, context) for every shape.
     static const bool split_only = [] {
         const char *e = std::getenv("CUBERT_ATTENTION");
         return e != nullptr && std::string(e) == "split";
     }();
-    if (!split_only) {
+    if (!split_only && fused_attention_fits) {
         Timed t(profiler, Profiler::kAttentionFused, stream);
         if (cuBERT::attention_fused(Q, K, V, ld, mask, context_out, H, alpha, B, A, S, d, stream)) return;
+        fused_attention_fits = false;  // seq_length and head size are fixed per model: do not ask again
     }
 
     const bool loop_heads = A <= B;

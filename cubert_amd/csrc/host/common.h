@@ -185,7 +185,7 @@ inline bool attention_context(const half *probs, const half *v, int ld, half *ct
     return true;
 }
 
-// The whole attention core (scores, mask, softmax, context) in one launch for seq_length <= 128; false when
+// The whole attention core (scores, mask, softmax, context) in one launch (seq_length <= 512); false when
 // the shape has no such kernel (reference: AttentionSelf.cpp:96-111 runs it as three operators).
 inline bool attention_fused(const float *q, const float *k, const float *v, int ld, const int8_t *mask, float *ctx,
                             int ld_ctx, float alpha, int batch, int heads, int seq, int head_size, void *stream) {

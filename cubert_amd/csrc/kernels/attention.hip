@@ -435,6 +435,186 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
     }
 }
 
+// ---- the same for longer sequences (128 < seq <= 512): online softmax over chunks of 64 keys ----
+// The layout is that of attention_fused_kernel (a workgroup per (batch, head), a wavefront per 32 queries, K and
+// slot-ordered V^T in LDS), but a lane cannot hold seq/2 scores, so the keys are walked in chunks: each chunk
+// updates the query's running maximum m and sum l, rescales the context accumulators by exp(m_old - m_new) and
+// adds exp(s - m_new) V.  The accumulators have queries along registers while m and l live in the lane of the
+// query, so the per-query factors cross lanes through 128 bytes of wavefront-private LDS.  The result is divided
+// by l once at the end (probabilities are not rounded to the storage type one by one as the three-kernel path
+// does; the difference is within the fp16 storage tolerance).
+template <typename T, int D>
+__global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restrict__ q, const T *__restrict__ k,
+                                                               const T *__restrict__ v, int ld,
+                                                               const int8_t *__restrict__ mask, T *__restrict__ ctx,
+                                                               int ld_ctx, float alpha, int heads, int seq) {
+    constexpr int V = Mma<T>::kVec;
+    constexpr int kSteps = D / 2 / V;
+    constexpr int kColTiles = D / 32;
+    constexpr int kChunk = 2;  // key tiles per step
+    constexpr int kPitchK = D + V;
+    const int S = seq, KT = seq / 32;
+    const int threads = blockDim.x;  // = KT * 64
+    const int pitch_v = S + V;
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *s_k = reinterpret_cast<T *>(smem);                              // [S][kPitchK]
+    T *s_vt = s_k + (size_t) S * kPitchK;                              // [D][pitch_v], keys in slot order
+    float *s_mask = reinterpret_cast<float *>(s_vt + (size_t) D * pitch_v);  // [S] additive mask
+    float *s_factor = s_mask + S;                                      // [KT][32] per-query factors
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int r = lane & 31, hh = lane >> 5;
+    const int qt = wave_in_block();
+    const int bh = blockIdx.x;
+    const int b = bh / heads, h = bh - b * heads;
+    const T *k_head = k + (size_t) b * S * ld + (size_t) h * D;
+    const T *v_head = v + (size_t) b * S * ld + (size_t) h * D;
+
+    const T *q_row = q + ((size_t) b * S + qt * 32 + r) * ld + (size_t) h * D + hh * (D / 2);
+    Vec<T, V> qv[kSteps];
+#pragma unroll
+    for (int t = 0; t < kSteps; ++t) qv[t] = load_vec<T, V>(q_row + t * V);
+
+    constexpr int kVecPerRow = D / V;
+    constexpr int kLoads = D / V / 2;  // vectors per thread for K, slot groups per thread for V^T
+    Vec<T, V> kreg[kLoads], vreg[kLoads];
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+        const int idx = threadIdx.x + u * threads;
+        const int row = idx / kVecPerRow, c = idx - row * kVecPerRow;
+        kreg[u] = load_vec<T, V>(k_head + (size_t) row * ld + c * V);
+    }
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+        const int idx = threadIdx.x + u * threads;
+        const int j = idx % D, grp = idx / D;
+        const int kt = grp / (32 / V), in_tile = grp % (32 / V);
+        const int run = in_tile >> 1, half = in_tile & 1;
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+            vreg[u].v[e] = v_head[(size_t) (kt * 32 + acc_row(run * V + e, half)) * ld + j];
+        }
+    }
+    for (int i = threadIdx.x; i < S; i += threads) {
+        s_mask[i] = (mask != nullptr && !mask[(size_t) b * S + i]) ? kMaskedScore : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+        const int idx = threadIdx.x + u * threads;
+        const int row = idx / kVecPerRow, c = idx - row * kVecPerRow;
+        store_vec<T, V>(s_k + row * kPitchK + c * V, kreg[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+        const int idx = threadIdx.x + u * threads;
+        const int j = idx % D, grp = idx / D;
+        store_vec<T, V>(s_vt + j * pitch_v + grp * V, vreg[u]);
+    }
+    __syncthreads();
+
+    float *factor = s_factor + qt * 32;  // private to this wavefront
+    float m = -3.402823466e+38f, l = 0.f;
+    v16f32 out[kColTiles];
+#pragma unroll
+    for (int jt = 0; jt < kColTiles; ++jt) out[jt] = v16f32{};
+
+    for (int c0 = 0; c0 < KT; c0 += kChunk) {
+        v16f32 p[kChunk];
+        float cm = -3.402823466e+38f;
+#pragma unroll
+        for (int cc = 0; cc < kChunk; ++cc) {
+            const int kt = c0 + cc;
+            v16f32 c = {};
+            if (kt < KT) {  // wavefront-uniform
+#pragma unroll
+                for (int t = 0; t < kSteps; ++t) {
+                    Mma<T>::run(c, load_vec<T, V>(s_k + (kt * 32 + r) * kPitchK + hh * (D / 2) + t * V), qv[t]);
+                }
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const Vec<float, 4> mk = load_vec<float, 4>(s_mask + kt * 32 + g * 8 + hh * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float sc = to_f32(from_f32<T>(c[g * 4 + e] * alpha)) + mk.v[e];
+                        c[g * 4 + e] = sc;
+                        cm = fmaxf(cm, sc);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) c[i] = -3.402823466e+38f;  // exp(. - m) = 0
+            }
+            p[cc] = c;
+        }
+        cm = fmaxf(cm, __shfl_xor(cm, 32, kWave));
+        const float m_new = fmaxf(m, cm);
+        const float f = __expf(m - m_new);  // 0 in the first chunk (m = -max float), where out is 0 anyway
+        float part = 0.f;
+#pragma unroll
+        for (int cc = 0; cc < kChunk; ++cc) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                p[cc][i] = __expf(p[cc][i] - m_new);
+                part += p[cc][i];
+            }
+        }
+        part += __shfl_xor(part, 32, kWave);
+        l = l * f + part;
+        m = m_new;
+
+        // rescale the accumulators: row i of a lane is query acc_row(i, hh), whose factor is in lane acc_row(i, hh)
+        if (c0 > 0) {
+            if (hh == 0) factor[r] = f;
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): LDS operations of one wavefront complete in order
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const Vec<float, 4> fr = load_vec<float, 4>(factor + g * 8 + hh * 4);
+#pragma unroll
+                for (int jt = 0; jt < kColTiles; ++jt) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) out[jt][g * 4 + e] *= fr.v[e];
+                }
+            }
+            __builtin_amdgcn_wave_barrier();  // the reads above come before the next chunk's write
+        }
+#pragma unroll
+        for (int cc = 0; cc < kChunk; ++cc) {
+            const int kt = c0 + cc;
+            if (kt < KT) {
+#pragma unroll
+                for (int run = 0; run < 16 / V; ++run) {
+                    Vec<T, V> a;
+#pragma unroll
+                    for (int e = 0; e < V; ++e) a.v[e] = from_f32<T>(p[cc][run * V + e]);
+#pragma unroll
+                    for (int jt = 0; jt < kColTiles; ++jt) {
+                        Mma<T>::run(out[jt], a,
+                                    load_vec<T, V>(s_vt + (jt * 32 + r) * pitch_v + kt * 32 + run * 2 * V + hh * V));
+                    }
+                }
+            }
+        }
+    }
+
+    // divide row (query) i by its sum
+    if (hh == 0) factor[r] = 1.f / l;
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_wave_barrier();
+    T *dst = ctx + ((size_t) b * S + qt * 32) * ld_ctx + (size_t) h * D + r;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const Vec<float, 4> fr = load_vec<float, 4>(factor + g * 8 + hh * 4);
+#pragma unroll
+        for (int jt = 0; jt < kColTiles; ++jt) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                dst[(size_t) acc_row(g * 4 + e, hh) * ld_ctx + jt * 32] = from_f32<T>(out[jt][g * 4 + e] * fr.v[e]);
+            }
+        }
+    }
+}
+
 template <typename T>
 bool shapes_ok(int batch, int heads, int seq, int head_size, int ld, std::initializer_list<const void *> ptrs) {
     constexpr int V = Mma<T>::kVec;
@@ -537,8 +717,8 @@ int launch_fused_kt(const T *q, const T *k, const T *v, int ld, const int8_t *ma
             raised = true;
         }
     }
-    return launch_lds(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask, ctx, ld_ctx,
-                      alpha, heads);
+    return launch_untimed(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask, ctx,
+                          ld_ctx, alpha, heads);
 }
 
 template <typename T, int D>
@@ -553,16 +733,45 @@ int launch_fused(const T *q, const T *k, const T *v, int ld, const int8_t *mask,
     }
 }
 
+template <typename T, int D>
+int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
+                 int batch, int heads, int seq, hipStream_t s) {
+    constexpr int V = 16 / sizeof(T);
+    if (seq > 512) return CUBERT_UNSUPPORTED;  // a workgroup has at most 16 wavefronts
+    const size_t lds = (size_t) seq * (D + V) * sizeof(T) + (size_t) D * (seq + V) * sizeof(T) +
+                       2 * (size_t) seq * sizeof(float);
+    if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
+    auto kernel = attention_flash_kernel<T, D>;
+    static thread_local bool raised = false;  // per instantiation and thread; the call is cheap and idempotent
+    if (!raised) {
+        if (hipFuncSetAttribute((const void *) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) !=
+            hipSuccess) {
+            (void) hipGetLastError();
+            return CUBERT_UNSUPPORTED;
+        }
+        raised = true;
+    }
+    return launch_untimed(kernel, dim3(batch * heads), dim3(seq / 32 * kWave), (unsigned) lds, s, q, k, v, ld, mask,
+                          ctx, ld_ctx, alpha, heads, seq);
+}
+
 template <typename T>
 int attention_fused(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
                     int batch, int heads, int seq, int head_size, void *stream) {
     if (batch == 0 || heads == 0 || seq == 0) return 0;
     if (!q || !k || !v || !ctx || batch < 0 || heads < 0 || seq < 0 || head_size <= 0) return CUBERT_BAD_ARGUMENT;
     if (ld < heads * head_size) return CUBERT_BAD_ARGUMENT;
-    if (seq > 128 || !shapes_ok<T>(batch, heads, seq, head_size, ld, {q, k, v}) || ld_ctx < heads * head_size) {
+    if (!shapes_ok<T>(batch, heads, seq, head_size, ld, {q, k, v}) || ld_ctx < heads * head_size) {
         return CUBERT_UNSUPPORTED;
     }
     hipStream_t s = (hipStream_t) stream;
+    if (seq > 128) {
+        switch (head_size) {
+            case 32: return launch_flash<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, s);
+            case 64: return launch_flash<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, s);
+            default: return CUBERT_UNSUPPORTED;  // head size 128 would spill the accumulators to scratch
+        }
+    }
     switch (head_size) {
         case 32: return launch_fused<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, s);
         case 64: return launch_fused<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, s);

@@ -121,6 +121,15 @@ inline int launch_lds(void (*kernel)(Params...), dim3 grid, dim3 block, unsigned
     return e == hipSuccess ? 0 : (int) e;
 }
 
+// A launch that never carries timing events (the pending pair, if any, stays pending for the next launch()).
+template <typename... Params, typename... Args>
+inline int launch_untimed(void (*kernel)(Params...), dim3 grid, dim3 block, unsigned lds_bytes, hipStream_t stream,
+                          Args... args) {
+    hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, static_cast<Params>(args)...);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : (int) e;
+}
+
 template <typename... Params, typename... Args>
 inline int launch(void (*kernel)(Params...), dim3 grid, dim3 block, hipStream_t stream, Args... args) {
     return launch_lds(kernel, grid, block, 0u, stream, args...);

@@ -90,7 +90,7 @@ def attention_scores(qkv, batch, heads, seq, head_size, alpha):
 
 
 def attention_fused(qkv, mask, batch, heads, seq, head_size, alpha):
-    """ctx[B*S, H] = softmax(alpha Q K^T + mask) V in one launch (seq <= 128); None when the shape does not fit."""
+    """ctx[B*S, H] = softmax(alpha Q K^T + mask) V in one launch (seq <= 512); None when the shape does not fit."""
     hidden = heads * head_size
     flat = qkv.view(-1)
     ctx = torch.empty((batch * seq, hidden), dtype=qkv.dtype, device=qkv.device)

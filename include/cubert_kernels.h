@@ -107,13 +107,15 @@ int cubert_attention_context_f32(const float *probs, const float *v, int ld, flo
 int cubert_attention_context_f16(const cubert_half *probs, const cubert_half *v, int ld, cubert_half *ctx, int ld_ctx,
                                  int batch, int heads, int seq_length, int head_size, void *stream);
 
-/* The attention core of one layer in a single launch, for seq_length <= 128:
+/* The attention core of one layer in a single launch:
  *   ctx[b, q, a, :] = sum_k softmax_k(alpha * Q[b,q,a,:] . K[b,k,a,:] + (mask[b,k] == 0 ? -10000 : 0)) * V[b, k, a, :]
- * with the [batch, heads, seq, seq] scores held in registers (never written to memory).  Scores and
- * probabilities are rounded to the storage type where the three-kernel sequence (cubert_attention_scores,
- * cubert_mask_scale_softmax, cubert_attention_context) stores them, so both give the same result up to
- * summation order.  mask may be NULL.  Same shape support as the two contractions, and seq_length <= 128;
- * anything else returns CUBERT_UNSUPPORTED and launches nothing.
+ * with the [batch, heads, seq, seq] scores held in registers (never written to memory).  Up to seq_length 128
+ * scores and probabilities are rounded to the storage type where the three-kernel sequence
+ * (cubert_attention_scores, cubert_mask_scale_softmax, cubert_attention_context) stores them, so both give the
+ * same result up to summation order; from 129 to 512 the softmax runs online over chunks of 64 keys and is
+ * normalised once at the end.  mask may be NULL.  Shape support as the two contractions, and seq_length <= 512
+ * (<= 128 for head_size 128, and K, V of one head must fit 160 KB of LDS: fp32 up to seq_length 256 at head size
+ * 64); anything else returns CUBERT_UNSUPPORTED and launches nothing.
  * replaces: AttentionSelf<T>::_in_compute's Att_Q_K -> Softmax -> Att_QK_V sequence and the mask tensor of
  * AttentionMask<T>::compute, reference src/cuBERT/op_att/AttentionSelf.cpp:96-111, AttentionMask.cpp:41-54. */
 int cubert_attention_fused_f32(const float *q, const float *k, const float *v, int ld, const int8_t *mask, float *ctx,

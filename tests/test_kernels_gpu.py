@@ -337,7 +337,9 @@ def test_attention_scores_and_context(K, name, batch, heads, seq, d):
 
 @pytest.mark.parametrize("name", ["f32", "f16"])
 @pytest.mark.parametrize("batch,heads,seq,d", [(3, 12, 32, 64), (2, 4, 128, 64), (2, 3, 64, 32), (1, 2, 96, 128),
-                                               (2, 16, 128, 64), (5, 1, 32, 64), (7, 3, 64, 64)])
+                                               (2, 16, 128, 64), (5, 1, 32, 64), (7, 3, 64, 64),
+                                               # longer than 128: the online-softmax kernel (chunks of 64 keys)
+                                               (1, 2, 512, 64), (2, 3, 256, 64), (2, 2, 160, 64), (1, 1, 384, 32)])
 @pytest.mark.parametrize("masked", [True, False])
 def test_attention_fused_against_oracle(K, name, batch, heads, seq, d, masked):
     """One-launch attention core vs the oracle's attention_self pieces (att_q_k -> mask -> softmax -> att_qk_v),
@@ -350,7 +352,9 @@ def test_attention_fused_against_oracle(K, name, batch, heads, seq, d, masked):
     mask[0, :] = 0
     alpha = 1.0 / math.sqrt(d)
     ctx = K.attention_fused(dev(qkv, tdt(name)), dev(mask) if masked else None, batch, heads, seq, d, alpha)
-    assert ctx is not None
+    if ctx is None:  # K and V of one head must fit 160 KB of LDS
+        assert seq * (d + 4) * 4 + d * (seq + 4) * 4 + 2 * seq * 4 > 160 * 1024 and name == "f32"
+        return
     scores = oracle.att_q_k(qh, kh, batch, seq, heads, d, alpha=alpha)  # [B, S_q, A, S_k]
     if name == "f16":
         scores = oracle.round_to_half(scores)  # the scaled scores are what is stored; the mask is added in fp32
@@ -385,8 +389,10 @@ def test_attention_unsupported_shapes_are_declined(K):
     assert K.attention_context(torch.zeros((2, 2, 4, 4), device="cuda"), qkv, 2, 2, 4, 3) is None
     qkv = torch.zeros((2 * 40, 3 * 128), device="cuda")
     assert K.attention_scores(qkv, 2, 2, 40, 64, 1.0) is None  # seq not a multiple of 32
-    qkv = torch.zeros((160, 3 * 128), device="cuda")
-    assert K.attention_fused(qkv, None, 1, 2, 160, 64, 1.0) is None   # longer than the fused kernel holds
+    qkv = torch.zeros((544, 3 * 128), device="cuda")
+    assert K.attention_fused(qkv, None, 1, 2, 544, 64, 1.0) is None   # more than 16 query tiles
+    qkv = torch.zeros((256, 3 * 256), device="cuda")
+    assert K.attention_fused(qkv, None, 1, 2, 256, 128, 1.0) is None  # long sequence with head size 128
 
 
 # ------------------------------------------------------------------ GEMM convention
