@@ -9,6 +9,7 @@ std::out_of_range -> IndexError.  Device errors terminate the process, as in the
 reference.
 """
 import ctypes
+import os
 
 import numpy as np
 
@@ -83,15 +84,94 @@ def _check_inputs(input_ids, input_mask, segment_ids):
     return input_ids.shape[0]
 
 
+def _text_array(texts):
+    """list of str/bytes -> (const char*[]) with the bytes objects kept alive by the returned pair."""
+    if texts is None:
+        return None, None
+    keep = [t.encode("utf8") if isinstance(t, str) else bytes(t) for t in texts]
+    return (ctypes.c_char_p * len(keep))(*keep), keep
+
+
+class Tokenizer(object):
+    """The text front end alone (CPU): the reference's FullTokenizer (src/cuBERT/tokenization.h:112-152), or with
+    vocab_file=None its BasicTokenizer."""
+
+    def __init__(self, vocab_file=None, do_lower_case=True):
+        self._h = None
+        self.do_lower_case = bool(do_lower_case)
+        if vocab_file is not None:
+            handle = ctypes.c_void_p()
+            _raise(lib().cubert_try_open_tokenizer(os.fsencode(vocab_file), int(self.do_lower_case),
+                                                   ctypes.byref(handle)))
+            self._h = handle
+
+    def close(self):
+        if self._h is not None:
+            lib().cuBERT_close_tokenizer(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @staticmethod
+    def _tokens(call):
+        n, needed = ctypes.c_int(), ctypes.c_size_t()
+        _raise(call(None, 0, ctypes.byref(n), ctypes.byref(needed)))
+        buf = ctypes.create_string_buffer(needed.value)
+        _raise(call(buf, needed.value, ctypes.byref(n), ctypes.byref(needed)))
+        return buf.value.decode("utf8").split("\n") if n.value else []
+
+    def tokenize(self, text, max_length=1 << 20):
+        """Word pieces of `text` (basic tokens when there is no vocabulary)."""
+        raw = text.encode("utf8") if isinstance(text, str) else bytes(text)
+        return self._tokens(lambda out, cap, n, needed: lib().cubert_tokenizer_tokenize(
+            self._h, int(self.do_lower_case), raw, max_length, out, cap, n, needed))
+
+    def wordpiece(self, token):
+        raw = token.encode("utf8") if isinstance(token, str) else bytes(token)
+        return self._tokens(lambda out, cap, n, needed: lib().cubert_tokenizer_wordpiece(self._h, raw, out, cap, n,
+                                                                                          needed))
+
+    def convert_tokens_to_ids(self, tokens):
+        return [int(lib().cubert_tokenizer_token_id(self._h, t.encode("utf8"))) for t in tokens]
+
+    def convert_example(self, max_seq_length, text_a, text_b=None):
+        """(input_ids int32, input_mask int8, segment_ids int8), each of max_seq_length entries."""
+        ids = np.zeros(max_seq_length, np.int32)
+        mask = np.zeros(max_seq_length, np.int8)
+        seg = np.zeros(max_seq_length, np.int8)
+        _raise(lib().cubert_tokenizer_convert_example(
+            self._h, max_seq_length, text_a.encode("utf8"), None if text_b is None else text_b.encode("utf8"),
+            ids.ctypes.data, mask.ctypes.data, seg.ctypes.data))
+        return ids, mask, seg
+
+
+def nfd(text):
+    """Canonical decomposition of a string by the library's own tables."""
+    raw = text.encode("utf8")
+    needed = ctypes.c_size_t()
+    _raise(lib().cubert_tokenizer_nfd(raw, None, 0, ctypes.byref(needed)))
+    buf = ctypes.create_string_buffer(needed.value)
+    _raise(lib().cubert_tokenizer_nfd(raw, buf, needed.value, ctypes.byref(needed)))
+    return buf.value.decode("utf8")
+
+
 class Model(object):
-    """A model opened from a frozen GraphDef file (cuBERT_open), one replica per visible GPU."""
+    """A model opened from a frozen GraphDef file (cuBERT_open), one replica per visible GPU; with a vocabulary
+    file also the tokenizer (cuBERT_open_tokenizer), as python/cuBERT.pyx:116-139 of the reference."""
 
     def __init__(self, model_file, max_batch_size, seq_length, num_hidden_layers, num_attention_heads,
                  compute_type=ComputeType.FLOAT, vocab_file=None, do_lower_case=1):
         self._c_model = None
+        self._c_tokenizer = None
         self._c_compute_type = compute_type
         if vocab_file:
-            raise ValueError("tokenizer is not part of this build: tokenize on the host and call compute")
+            handle = ctypes.c_void_p()
+            _raise(lib().cubert_try_open_tokenizer(os.fsencode(vocab_file), int(do_lower_case), ctypes.byref(handle)))
+            self._c_tokenizer = handle
         if isinstance(model_file, str):
             model_file = model_file.encode("utf8")
         handle = ctypes.c_void_p()
@@ -106,6 +186,9 @@ class Model(object):
         if self._c_model is not None:
             _raise(lib().cubert_try_close(self._c_model, self._c_compute_type))
             self._c_model = None
+        if self._c_tokenizer is not None:
+            lib().cuBERT_close_tokenizer(self._c_tokenizer)
+            self._c_tokenizer = None
 
     def __del__(self):
         try:
@@ -129,6 +212,32 @@ class Model(object):
         _raise(lib().cubert_try_compute_m(self._c_model, batch, input_ids.ctypes.data, input_mask.ctypes.data,
                                           segment_ids.ctypes.data, ctypes.byref(output._c), self._c_compute_type,
                                           int(bool(output_to_float))))
+
+
+    def tokenize_compute(self, text_a, text_b, output, output_type=OutputType.LOGITS):
+        """Texts in, one output array out (python/cuBERT.pyx:181-189)."""
+        if self._c_tokenizer is None:
+            raise ValueError("the model was opened without a vocab_file")
+        if text_b is not None and len(text_a) != len(text_b):
+            raise ValueError("text_a and text_b differ in length")
+        if not isinstance(output, np.ndarray) or not output.flags["C_CONTIGUOUS"]:
+            raise ValueError("numpy array should be C_CONTIGUOUS")
+        a, keep_a = _text_array(text_a)
+        b, keep_b = _text_array(text_b)
+        _raise(lib().cubert_try_tokenize_compute(self._c_model, self._c_tokenizer, len(keep_a), a, b,
+                                                 output.ctypes.data, output_type, self._c_compute_type))
+
+    def tokenize_compute_m(self, text_a, text_b, output, output_to_float=False):
+        """Texts in, several outputs out (python/cuBERT.pyx:191-208)."""
+        if self._c_tokenizer is None:
+            raise ValueError("the model was opened without a vocab_file")
+        if text_b is not None and len(text_a) != len(text_b):
+            raise ValueError("text_a and text_b differ in length")
+        a, keep_a = _text_array(text_a)
+        b, keep_b = _text_array(text_b)
+        _raise(lib().cubert_try_tokenize_compute_m(self._c_model, self._c_tokenizer, len(keep_a), a, b,
+                                                   ctypes.byref(output._c), self._c_compute_type,
+                                                   int(bool(output_to_float))))
 
 
 class Bert(object):

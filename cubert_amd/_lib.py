@@ -43,6 +43,18 @@ SIGNATURES = {
     "cubert_try_compute_m": (ci, [vp, ci, vp, vp, vp, ctypes.POINTER(cuBERT_Output), ci, ci]),
     "cubert_try_close": (ci, [vp, ci]),
     "cubert_model_info": (ci, [vp, ci, ctypes.POINTER(ci), ctypes.POINTER(ci), ctypes.POINTER(ci)]),
+    "cubert_try_open_tokenizer": (ci, [ctypes.c_char_p, ci, ctypes.POINTER(vp)]),
+    "cubert_try_tokenize_compute": (ci, [vp, vp, ci, vp, vp, vp, ci, ci]),
+    "cubert_try_tokenize_compute_m": (ci, [vp, vp, ci, vp, vp, ctypes.POINTER(cuBERT_Output), ci, ci]),
+    "cubert_tokenizer_tokenize": (ci, [vp, ci, ctypes.c_char_p, ci, vp, ctypes.c_size_t, ctypes.POINTER(ci),
+                                       ctypes.POINTER(ctypes.c_size_t)]),
+    "cubert_tokenizer_wordpiece": (ci, [vp, ctypes.c_char_p, vp, ctypes.c_size_t, ctypes.POINTER(ci),
+                                        ctypes.POINTER(ctypes.c_size_t)]),
+    "cubert_tokenizer_token_id": (ctypes.c_longlong, [vp, ctypes.c_char_p]),
+    "cubert_tokenizer_convert_example": (ci, [vp, ci, ctypes.c_char_p, ctypes.c_char_p, vp, vp, vp]),
+    "cubert_tokenizer_char_class": (ci, [ci, ci]),
+    "cubert_tokenizer_nfd": (ci, [ctypes.c_char_p, vp, ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t)]),
+    "cubert_tokenizer_unicode_version": (ctypes.c_char_p, []),
     "cubert_bert_create": (ci, [ci, ci, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(vp), ci, ci, ci, ci, ci, ci, ci,
                                 ci, ci, ctypes.POINTER(vp)]),
     "cubert_bert_compute": (ci, [vp, ci, ci, vp, vp, vp]),

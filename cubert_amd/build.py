@@ -25,7 +25,8 @@ HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-a
 
 DEVICE_SOURCES = ["kernels/layernorm.hip", "kernels/softmax.hip", "kernels/elementwise.hip", "kernels/attention.hip", "kernels/gemm_skinny.hip",
                   "runtime.hip"]
-HOST_SOURCES = ["host/Transformer.cpp", "host/Bert.cpp", "host/BertM.cpp", "host/Graph.cpp", "host/api.cpp"]
+HOST_SOURCES = ["host/Transformer.cpp", "host/Bert.cpp", "host/BertM.cpp", "host/Graph.cpp", "host/tokenization.cpp",
+                "host/api.cpp"]
 
 
 def hipcc():

@@ -1,13 +1,16 @@
 // The public C API (include/cuBERT.h) and the exception-free host entry points
 // (include/cubert_host.h).
+#include <cstring>
 #include <stdexcept>
 #include <string>
 #include <unordered_map>
+#include <vector>
 
 #include "Bert.h"
 #include "BertM.h"
 #include "Transformer.h"
 #include "cuBERT.h"
+#include "tokenization.h"
 #include "cubert_host.h"
 
 using cuBERT::half;
@@ -58,22 +61,56 @@ void cuBERT_close(void *model, cuBERT_ComputeType compute_type) {
     }
 }
 
-// The WordPiece tokenizer is host-side string processing outside the device path this library
-// replaces; the symbols exist so that binaries linked against the reference still resolve.
-void *cuBERT_open_tokenizer(const char *, int) {
-    throw std::invalid_argument("tokenizer is not part of this build: tokenize on the host and call cuBERT_compute");
+void *cuBERT_open_tokenizer(const char *vocab_file, int do_lower_case) {
+    return new cuBERT::FullTokenizer(vocab_file, do_lower_case != 0);
 }
 
-void cuBERT_close_tokenizer(void *) {}
+void cuBERT_close_tokenizer(void *tokenizer) { delete (cuBERT::FullTokenizer *) tokenizer; }
 
-void cuBERT_tokenize_compute(void *, void *, int, const char **, const char **, void *, cuBERT_OutputType,
-                             cuBERT_ComputeType) {
-    throw std::invalid_argument("tokenizer is not part of this build: tokenize on the host and call cuBERT_compute");
+namespace {
+
+size_t model_seq_length(void *model, cuBERT_ComputeType compute_type) {
+    if (model == nullptr) throw std::invalid_argument("null model");
+    return compute_type == cuBERT_COMPUTE_FLOAT ? ((cuBERT::BertM<float> *) model)->seq_length
+                                                : ((cuBERT::BertM<half> *) model)->seq_length;
 }
 
-void cuBERT_tokenize_compute_m(void *, void *, int, const char **, const char **, cuBERT_Output *, cuBERT_ComputeType,
-                               int) {
-    throw std::invalid_argument("tokenizer is not part of this build: tokenize on the host and call cuBERT_compute_m");
+// text -> ids, mask, segment ids for a batch (reference: cuBERT.cpp:216-247; heap instead of stack arrays)
+struct TokenizedBatch {
+    std::vector<int> input_ids;
+    std::vector<int8_t> input_mask, segment_ids;
+
+    TokenizedBatch(void *tokenizer, size_t seq_length, int batch_size, const char **text_a, const char **text_b) {
+        if (tokenizer == nullptr || batch_size < 0 || (batch_size > 0 && text_a == nullptr)) {
+            throw std::invalid_argument("tokenizer, text_a and a non-negative batch_size are required");
+        }
+        const size_t n = (size_t) batch_size * seq_length;
+        input_ids.resize(n);
+        input_mask.resize(n);
+        segment_ids.resize(n);
+        const auto *tok = (const cuBERT::FullTokenizer *) tokenizer;
+        for (int i = 0; i < batch_size; ++i) {
+            tok->convert_single_example(seq_length, text_a[i], text_b == nullptr ? nullptr : text_b[i],
+                                        input_ids.data() + seq_length * i, input_mask.data() + seq_length * i,
+                                        segment_ids.data() + seq_length * i);
+        }
+    }
+};
+
+}  // namespace
+
+void cuBERT_tokenize_compute(void *model, void *tokenizer, int batch_size, const char **text_a, const char **text_b,
+                             void *output, cuBERT_OutputType output_type, cuBERT_ComputeType compute_type) {
+    TokenizedBatch t(tokenizer, model_seq_length(model, compute_type), batch_size, text_a, text_b);
+    cuBERT_compute(model, batch_size, t.input_ids.data(), t.input_mask.data(), t.segment_ids.data(), output,
+                   output_type, compute_type);
+}
+
+void cuBERT_tokenize_compute_m(void *model, void *tokenizer, int batch_size, const char **text_a, const char **text_b,
+                               cuBERT_Output *output, cuBERT_ComputeType compute_type, int output_to_float) {
+    TokenizedBatch t(tokenizer, model_seq_length(model, compute_type), batch_size, text_a, text_b);
+    cuBERT_compute_m(model, batch_size, t.input_ids.data(), t.input_mask.data(), t.segment_ids.data(), output,
+                     compute_type, output_to_float);
 }
 
 // ------------------------------------------------------------- cubert_host.h
@@ -165,6 +202,126 @@ int cubert_try_compute_m(void *model, int batch_size, int *input_ids, int8_t *in
 int cubert_try_close(void *model, int compute_type) {
     return guarded([&] { cuBERT_close(model, (cuBERT_ComputeType) compute_type); });
 }
+
+namespace {
+
+// tokens joined by '\n' into a caller buffer
+void emit_tokens(const std::vector<std::string> &tokens, const char *sep, char *out, size_t capacity, int *n_tokens,
+                 size_t *needed) {
+    size_t bytes = 1;
+    for (const auto &t : tokens) bytes += t.size();
+    if (!tokens.empty()) bytes += (tokens.size() - 1) * std::strlen(sep);
+    if (n_tokens) *n_tokens = (int) tokens.size();
+    if (needed) *needed = bytes;
+    if (out == nullptr || capacity < bytes) return;
+    char *p = out;
+    for (size_t i = 0; i < tokens.size(); ++i) {
+        if (i) {
+            std::memcpy(p, sep, std::strlen(sep));
+            p += std::strlen(sep);
+        }
+        std::memcpy(p, tokens[i].data(), tokens[i].size());
+        p += tokens[i].size();
+    }
+    *p = 0;
+}
+
+}  // namespace
+
+int cubert_try_open_tokenizer(const char *vocab_file, int do_lower_case, void **tokenizer) {
+    return guarded([&] {
+        if (vocab_file == nullptr || tokenizer == nullptr) throw std::invalid_argument("null argument");
+        *tokenizer = cuBERT_open_tokenizer(vocab_file, do_lower_case);
+    });
+}
+
+int cubert_try_tokenize_compute(void *model, void *tokenizer, int batch_size, const char **text_a, const char **text_b,
+                                void *output, int output_type, int compute_type) {
+    return guarded([&] {
+        cuBERT_tokenize_compute(model, tokenizer, batch_size, text_a, text_b, output, (cuBERT_OutputType) output_type,
+                                (cuBERT_ComputeType) compute_type);
+    });
+}
+
+int cubert_try_tokenize_compute_m(void *model, void *tokenizer, int batch_size, const char **text_a,
+                                  const char **text_b, cuBERT_Output *output, int compute_type, int output_to_float) {
+    return guarded([&] {
+        cuBERT_tokenize_compute_m(model, tokenizer, batch_size, text_a, text_b, output,
+                                  (cuBERT_ComputeType) compute_type, output_to_float);
+    });
+}
+
+int cubert_tokenizer_tokenize(void *tokenizer, int do_lower_case, const char *text, int max_length, char *out,
+                              size_t capacity, int *n_tokens, size_t *needed) {
+    return guarded([&] {
+        if (text == nullptr || max_length < 0) throw std::invalid_argument("text and a non-negative max_length are required");
+        std::vector<std::string> tokens;
+        if (tokenizer != nullptr) {
+            ((const cuBERT::FullTokenizer *) tokenizer)->tokenize(text, &tokens, (size_t) max_length);
+        } else {
+            cuBERT::BasicTokenizer(do_lower_case != 0).tokenize(text, &tokens, (size_t) max_length);
+        }
+        emit_tokens(tokens, "\n", out, capacity, n_tokens, needed);
+    });
+}
+
+int cubert_tokenizer_wordpiece(void *tokenizer, const char *token, char *out, size_t capacity, int *n_tokens,
+                               size_t *needed) {
+    return guarded([&] {
+        if (tokenizer == nullptr || token == nullptr) throw std::invalid_argument("null argument");
+        std::vector<std::string> tokens;
+        ((const cuBERT::FullTokenizer *) tokenizer)->wordpiece(token, &tokens);
+        emit_tokens(tokens, "\n", out, capacity, n_tokens, needed);
+    });
+}
+
+long long cubert_tokenizer_token_id(void *tokenizer, const char *token) {
+    if (tokenizer == nullptr || token == nullptr) return 0;
+    return (long long) ((const cuBERT::FullTokenizer *) tokenizer)->convert_token_to_id(token);
+}
+
+int cubert_tokenizer_convert_example(void *tokenizer, int max_seq_length, const char *text_a, const char *text_b,
+                                     int *input_ids, int8_t *input_mask, int8_t *segment_ids) {
+    return guarded([&] {
+        if (!tokenizer || !text_a || !input_ids || !input_mask || !segment_ids || max_seq_length < 0) {
+            throw std::invalid_argument("null argument");
+        }
+        ((const cuBERT::FullTokenizer *) tokenizer)->convert_single_example((size_t) max_seq_length, text_a, text_b,
+                                                                            input_ids, input_mask, segment_ids);
+    });
+}
+
+int cubert_tokenizer_char_class(int which, int code_point) {
+    switch (which) {
+        case 0: return cuBERT::_is_whitespace(code_point);
+        case 1: return cuBERT::_is_control(code_point);
+        case 2: return cuBERT::_is_punctuation(code_point);
+        default: return -1;
+    }
+}
+
+int cubert_tokenizer_nfd(const char *text, char *out, size_t capacity, size_t *needed) {
+    return guarded([&] {
+        if (text == nullptr) throw std::invalid_argument("null text");
+        std::vector<uint32_t> cps, decomposed;
+        const unsigned char *s = (const unsigned char *) text;
+        size_t left = std::strlen(text);
+        while (left > 0) {
+            uint32_t cp;
+            const int len = cuBERT::unicode::decode_utf8(s, left, &cp);
+            if (len < 0) throw std::invalid_argument("malformed UTF-8");
+            cps.push_back(cp);
+            s += len;
+            left -= (size_t) len;
+        }
+        cuBERT::unicode::nfd(cps, &decomposed);
+        std::vector<std::string> one(1);
+        for (uint32_t cp : decomposed) cuBERT::unicode::append_utf8(cp, &one[0]);
+        emit_tokens(one, "", out, capacity, nullptr, needed);
+    });
+}
+
+const char *cubert_tokenizer_unicode_version(void) { return cuBERT::unicode::version(); }
 
 int cubert_model_info(void *model, int compute_type, int *hidden_size, int *num_labels, int *seq_length) {
     return guarded([&] {

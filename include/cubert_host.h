@@ -54,6 +54,40 @@ int cubert_try_compute_m(void *model, int batch_size, int *input_ids, int8_t *in
 int cubert_try_close(void *model, int compute_type);
 /* Shape facts of an opened model (hidden size, labels, seq_length) for sizing output arrays. */
 int cubert_model_info(void *model, int compute_type, int *hidden_size, int *num_labels, int *seq_length);
+/* replaces: cuBERT_open_tokenizer, reference src/cuBERT.cpp:104-106 */
+int cubert_try_open_tokenizer(const char *vocab_file, int do_lower_case, void **tokenizer);
+/* replaces: cuBERT_tokenize_compute / cuBERT_tokenize_compute_m, reference src/cuBERT.cpp:216-280 */
+int cubert_try_tokenize_compute(void *model, void *tokenizer, int batch_size, const char **text_a, const char **text_b,
+                                void *output, int output_type, int compute_type);
+int cubert_try_tokenize_compute_m(void *model, void *tokenizer, int batch_size, const char **text_a,
+                                  const char **text_b, cuBERT_Output *output, int compute_type, int output_to_float);
+
+/* ---- 1b. the tokenizer by itself (CPU only; no counterpart in the reference's C API, which reaches these
+ *          only through cuBERT_tokenize_compute) ---------------------------------------------------------- */
+
+/* FullTokenizer::tokenize (reference src/cuBERT/tokenization.cpp:218-228), or with tokenizer == NULL
+ * BasicTokenizer(do_lower_case)::tokenize (tokenization.cpp:116-183).  The tokens are written to `out` separated
+ * by '\n' (a token never contains white space) and NUL terminated; *n_tokens receives their number and *needed
+ * the bytes required including the NUL.  When `capacity` is too small nothing is written and the call still
+ * returns 0: call again with a buffer of *needed bytes. */
+int cubert_tokenizer_tokenize(void *tokenizer, int do_lower_case, const char *text, int max_length, char *out,
+                              size_t capacity, int *n_tokens, size_t *needed);
+/* WordpieceTokenizer::tokenize on one basic token (tokenization.cpp:186-216); output as above. */
+int cubert_tokenizer_wordpiece(void *tokenizer, const char *token, char *out, size_t capacity, int *n_tokens,
+                               size_t *needed);
+/* FullTokenizer::convert_token_to_id (tokenization.h:131-139): 0 and a message on stderr for an unknown token. */
+long long cubert_tokenizer_token_id(void *tokenizer, const char *token);
+/* convert_single_example (src/cuBERT.cpp:137-214): [CLS] a [SEP] (b [SEP]) -> ids, mask, segment ids, padded
+ * to max_seq_length entries each.  text_b may be NULL. */
+int cubert_tokenizer_convert_example(void *tokenizer, int max_seq_length, const char *text_a, const char *text_b,
+                                     int *input_ids, int8_t *input_mask, int8_t *segment_ids);
+/* _is_whitespace / _is_control / _is_punctuation (tokenization.cpp:84-94): which = 0 / 1 / 2. */
+int cubert_tokenizer_char_class(int which, int code_point);
+/* NFD of a UTF-8 string (what utf8proc_NFD gives the reference, tokenization.cpp:123-125); output as for
+ * cubert_tokenizer_tokenize without separators.  Returns 1 (invalid argument) for malformed UTF-8. */
+int cubert_tokenizer_nfd(const char *text, char *out, size_t capacity, size_t *needed);
+/* Version of the Unicode database the tables were generated from, e.g. "13.0.0". */
+const char *cubert_tokenizer_unicode_version(void);
 
 /* ---- 2. host classes ------------------------------------------------------- */
 

@@ -211,6 +211,49 @@ def test_open_half_and_output_to_float(cb, small_pb):
     assert_close(o.pooled_output, want["pooled_output"], FP16_TOL)
 
 
+def test_tokenize_compute(cb, small_pb, tmp_path):
+    """cuBERT_tokenize_compute(_m) (reference: src/cuBERT.cpp:216-280, test/cuBERT_test.cpp:58-107): texts in,
+    outputs equal to cuBERT_compute on the ids the oracle's convert_single_example gives, and to the oracle's
+    forward pass on them.  The vocabulary is made of characters and word pieces with ids inside the small
+    model's 211-row embedding table."""
+    from oracle import tokenizer as otok
+    path, w = small_pb
+    lines = ["[PAD]", "[UNK]", "[CLS]", "[SEP]"] + list("abcdefghijklmnopqrstuvwxyz0123456789,.!?") + \
+            ["##" + c for c in "abcdefghijklmnopqrstuvwxyz"] + ["the", "##ing", "run", "知", "乎", "在", "家", "刷"]
+    assert len(lines) < SMALL["vocab"]
+    vocab_path = tmp_path / "vocab.txt"
+    vocab_path.write_text("\n".join(lines) + "\n", encoding="utf8")
+    vocab = otok.load_vocab(lines)
+    text_a = ["知乎", "The running DOG, again!", "x", "Ünïcödé and more and more and more words than fit in here ok"]
+    text_b = ["在家刷知乎", "what?", "", "second part that is also rather long, to force truncation of both"]
+    model = cb.Model(path, 8, 32, 3, 4, vocab_file=str(vocab_path))
+    for b in (text_b, None):
+        feats = [otok.convert_single_example(vocab, 32, a, None if b is None else b[i]) for i, a in enumerate(text_a)]
+        ids = np.array([f[0] for f in feats], np.int32)
+        mask = np.array([f[1] for f in feats], np.int8)
+        seg = np.array([f[2] for f in feats], np.int8)
+        want = oracle.bert_forward(w, ids, mask, seg, 3, 4)
+        direct = np.zeros((4, 2), np.float32)
+        model.compute(ids, mask, seg, direct, cb.OutputType.LOGITS)
+        out = np.zeros((4, 2), np.float32)
+        model.tokenize_compute(text_a, b, out, cb.OutputType.LOGITS)
+        assert np.array_equal(out, direct)
+        assert_close(out, want["logits"], FP32_TOL, "tokenize_compute logits")
+        o = cb.Output()
+        o.probs = np.zeros((4, 2), np.float32)
+        o.pooled_output = np.zeros((4, 128), np.float32)
+        model.tokenize_compute_m(text_a, b, o)
+        assert_close(o.probs, want["probs"], FP32_TOL, "tokenize_compute_m probs")
+        assert_close(o.pooled_output, want["pooled_output"], FP32_TOL, "tokenize_compute_m pooled")
+    with pytest.raises(ValueError):
+        model.tokenize_compute(text_a, text_b[:2], np.zeros((4, 2), np.float32))
+    model.close()
+    plain = cb.Model(path, 8, 32, 3, 4)
+    with pytest.raises(ValueError, match="vocab_file"):
+        plain.tokenize_compute(text_a, None, np.zeros((4, 2), np.float32))
+    plain.close()
+
+
 def test_api_error_behaviour(cb, small_pb):
     path, _ = small_pb
     with pytest.raises(ValueError, match="model file not found"):
