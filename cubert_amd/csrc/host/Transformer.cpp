@@ -201,13 +201,21 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
                                 w.attention_norm_gamma, stream);
         }
 
-        // intermediate: dense (bias deferred), then bias + GELU
-        {
+        // intermediate: dense (bias deferred), then bias + GELU; one launch for both at <= 32 tokens
+        bool intermediate_done = false;
+        if (M <= 32 && dense_gelu_fits) {
             Timed t(profiler, Profiler::kDenseGemm, stream);
-            cuBERT::blas_gemm(cublas, false, false, I, M, H, 1.f, w.intermediate_kernel, I, attention_output, H, 0.f,
-                              intermediate_output, I);
+            intermediate_done = cuBERT::dense_gelu_few_tokens(cublas, I, M, H, w.intermediate_kernel, I,
+                                                              attention_output, H, intermediate_output, I,
+                                                              w.intermediate_bias);
+            dense_gelu_fits = intermediate_done;  // the layer sizes are fixed per model: do not ask again
         }
-        {
+        if (!intermediate_done) {
+            {
+                Timed t(profiler, Profiler::kDenseGemm, stream);
+                cuBERT::blas_gemm(cublas, false, false, I, M, H, 1.f, w.intermediate_kernel, I, attention_output, H,
+                                  0.f, intermediate_output, I);
+            }
             Timed t(profiler, Profiler::kBiasGelu, stream);
             cuBERT::gelu(intermediate_output, w.intermediate_bias, M, I, stream);
         }

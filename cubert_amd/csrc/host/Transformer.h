@@ -64,6 +64,7 @@ private:
 
     void *cublas;
     Profiler *profiler = nullptr;
+    bool dense_gelu_fits = true;       // cleared when the few-token Dense + GELU kernel declines this model's shape
     bool fused_attention_fits = true;  // cleared when the one-launch attention kernel declines this model's shape
     size_t max_batch_size, seq_length, hidden_size, num_hidden_layers, num_attention_heads, intermediate_size;
 

@@ -82,6 +82,23 @@ inline void blas_gemm(void *handle, bool TransA, bool TransB, int M, int N, int 
                       const half *B, int ldb, float beta, half *C, int ldc, const half *bias = nullptr) {
     CUBERT_CHECK(cubert_gemm_f16(handle, TransA, TransB, M, N, K, alpha, h(A), lda, h(B), ldb, beta, h(C), ldc, h(bias)));
 }
+// Dense + bias + GELU in one launch for at most 32 tokens (column-major C[M, N] = gelu(A B + bias), N <= 32);
+// false when the few-token kernel does not take the problem (the caller then runs blas_gemm and gelu).
+inline bool dense_gelu_few_tokens(void *handle, int M, int N, int K, const float *A, int lda, const float *B, int ldb,
+                                  float *C, int ldc, const float *bias) {
+    const int rc = cubert_gemm_skinny_f32(handle, M, N, K, 1.f, A, lda, B, ldb, C, ldc, bias, 1);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+inline bool dense_gelu_few_tokens(void *handle, int M, int N, int K, const half *A, int lda, const half *B, int ldb,
+                                  half *C, int ldc, const half *bias) {
+    const int rc = cubert_gemm_skinny_f16(handle, M, N, K, 1.f, h(A), lda, h(B), ldb, h(C), ldc, h(bias), 1);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+
 inline void blas_gemm_strided_batch(void *handle, bool TransA, bool TransB, int m, int n, int k, float alpha,
                                     const float *A, int lda, long long strideA, const float *B, int ldb,
                                     long long strideB, float beta, float *C, int ldc, long long strideC,

@@ -15,6 +15,7 @@
 // workspace and the last workgroup to arrive for a feature block (ticket from an atomic counter) adds the
 // slices in slice order, so the result does not depend on scheduling.
 
+#include "activations.h"
 #include "cubert_kernels.h"
 #include "device_common.h"
 
@@ -30,7 +31,7 @@ constexpr int kSkinnyChunk = 16;  // reduction values a wavefront consumes per p
 // Accumulator register i of the lane half hh holds this row of a 32x32 MFMA result (column = lane % 32).
 __device__ __forceinline__ int acc_row(int i, int hh) { return (i >> 2) * 8 + hh * 4 + (i & 3); }
 
-template <typename T>
+template <typename T, bool GELU>
 __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__restrict__ A, int lda,
                                                                      const T *__restrict__ B, int ldb,
                                                                      const T *__restrict__ bias, T *__restrict__ C,
@@ -94,16 +95,16 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
         if (*ticket != slices - 1) return;
         // last workgroup of this feature block: every slice's partial tile is complete
         sum = 0.f;
-        for (int s0 = 0; s0 < slices; s0 += 4) {  // four loads in flight, added in slice order
-            float p[4];
+        for (int s0 = 0; s0 < slices; s0 += 16) {  // up to 16 loads in flight, added in slice order
+            float p[16];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < 16; ++u) {
                 p[u] = s0 + u < slices ? __hip_atomic_load(&partials[((size_t) (s0 + u) * 32 + token) * pitch + m0 + f],
                                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
                                        : 0.f;
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) sum += p[u];
+            for (int u = 0; u < 16; ++u) sum += p[u];
         }
         if (threadIdx.x == 0) {  // ready for the next launch
             __hip_atomic_store(&counters[blockIdx.x], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -112,6 +113,7 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
     if (live) {
         float v = alpha * sum;
         if (bias != nullptr) v += to_f32(bias[m0 + f]);
+        if (GELU) v = GeluOp<T>()(v);
         C[(size_t) token * ldc + m0 + f] = from_f32<T>(v);
     }
 }
@@ -119,11 +121,13 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
 }  // namespace
 
 // Launches the kernel when the problem fits it, else returns CUBERT_UNSUPPORTED and launches nothing.
+// activation: 0 = none, 1 = erf-form GELU applied to alpha * A B + bias (the BertIntermediate layer).
 // `partials` holds partial_floats floats, `counters` n_counters ints that are zero between launches.
 template <typename T>
 int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, const T *B, int ldb, T *C, int ldc,
-                const T *bias, float *partials, size_t partial_floats, int *counters, int n_counters,
-                hipStream_t stream) {
+                const T *bias, int activation, float *partials, size_t partial_floats, int *counters,
+                int n_counters, hipStream_t stream) {
+    if (activation != 0 && activation != 1) return CUBERT_BAD_ARGUMENT;
     if (M <= 0 || N <= 0 || N > 32 || K <= 0 || K % kSkinnyChunk != 0) return CUBERT_UNSUPPORTED;
     if (lda < M || ldb < K || ldc < M) return CUBERT_BAD_ARGUMENT;
     if (!is_aligned(B, 16) || (ldb * sizeof(T)) % 16 != 0) return CUBERT_UNSUPPORTED;
@@ -137,13 +141,18 @@ int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, const T *
         slices = (chunks + chunks_per_slice - 1) / chunks_per_slice;
     }
     if (blocks > 65535 || slices > 65535 || (slices > 1 && blocks > n_counters)) return CUBERT_UNSUPPORTED;
-    return launch(gemm_skinny_kernel<T>, dim3(blocks, slices), dim3(kSkinnyThreads), stream, A, lda, B, ldb, bias, C,
-                  ldc, M, N, K, alpha, partials, counters, chunks_per_slice);
+    const dim3 grid(blocks, slices), block(kSkinnyThreads);
+    if (activation == 1) {
+        return launch(gemm_skinny_kernel<T, true>, grid, block, stream, A, lda, B, ldb, bias, C, ldc, M, N, K, alpha,
+                      partials, counters, chunks_per_slice);
+    }
+    return launch(gemm_skinny_kernel<T, false>, grid, block, stream, A, lda, B, ldb, bias, C, ldc, M, N, K, alpha,
+                  partials, counters, chunks_per_slice);
 }
 
 template int gemm_skinny<float>(int, int, int, float, const float *, int, const float *, int, float *, int,
-                                const float *, float *, size_t, int *, int, hipStream_t);
+                                const float *, int, float *, size_t, int *, int, hipStream_t);
 template int gemm_skinny<half_t>(int, int, int, float, const half_t *, int, const half_t *, int, half_t *, int,
-                                 const half_t *, float *, size_t, int *, int, hipStream_t);
+                                 const half_t *, int, float *, size_t, int *, int, hipStream_t);
 
 }  // namespace cubert

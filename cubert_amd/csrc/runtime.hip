@@ -25,8 +25,8 @@ namespace cubert {
 // kernels/gemm_skinny.hip
 template <typename T>
 int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, const T *B, int ldb, T *C, int ldc,
-                const T *bias, float *partials, size_t partial_floats, int *counters, int n_counters,
-                hipStream_t stream);
+                const T *bias, int activation, float *partials, size_t partial_floats, int *counters,
+                int n_counters, hipStream_t stream);
 
 LaunchTiming &pending_launch_timing() {
     static thread_local LaunchTiming pending;
@@ -212,15 +212,15 @@ bool library_gemm_only() {
 }
 
 int run_skinny(BlasContext *ctx, int type, int M, int N, int K, float alpha, const void *A, int lda, const void *B,
-               int ldb, void *C, int ldc, const void *bias) {
+               int ldb, void *C, int ldc, const void *bias, int activation) {
     if (type == 0) {
         return cubert::gemm_skinny<float>(M, N, K, alpha, (const float *) A, lda, (const float *) B, ldb, (float *) C,
-                                          ldc, (const float *) bias, ctx->skinny_partials, kSkinnyPartialFloats,
-                                          ctx->skinny_counters, kSkinnyCounters, ctx->stream);
+                                          ldc, (const float *) bias, activation, ctx->skinny_partials,
+                                          kSkinnyPartialFloats, ctx->skinny_counters, kSkinnyCounters, ctx->stream);
     }
     return cubert::gemm_skinny<cubert::half_t>(M, N, K, alpha, (const cubert::half_t *) A, lda,
                                                (const cubert::half_t *) B, ldb, (cubert::half_t *) C, ldc,
-                                               (const cubert::half_t *) bias, ctx->skinny_partials,
+                                               (const cubert::half_t *) bias, activation, ctx->skinny_partials,
                                                kSkinnyPartialFloats, ctx->skinny_counters, kSkinnyCounters,
                                                ctx->stream);
 }
@@ -238,7 +238,7 @@ int run_gemm(void *handle, int type, int transA, int transB, int M, int N, int K
                               beta, C, ldc, strideC, batch, bias);
     }
     if (!transA && !transB && batch == 1 && beta == 0.f && N <= 32 && !library_gemm_only()) {
-        const int rc = run_skinny(ctx, type, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias);
+        const int rc = run_skinny(ctx, type, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, 0);
         if (rc != CUBERT_UNSUPPORTED) return rc;
     }
     std::lock_guard<std::mutex> lock(ctx->mutex);
@@ -403,17 +403,20 @@ int cubert_gemm_f16(void *handle, int transA, int transB, int M, int N, int K, f
 }
 
 int cubert_gemm_skinny_f32(void *handle, int M, int N, int K, float alpha, const float *A, int lda, const float *B,
-                           int ldb, float *C, int ldc, const float *bias) {
+                           int ldb, float *C, int ldc, const float *bias, int activation) {
     BlasContext *ctx = (BlasContext *) handle;
     if (!ctx || !A || !B || !C) return CUBERT_BAD_ARGUMENT;
-    return run_skinny(ctx, 0, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias);
+    if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;
+    return run_skinny(ctx, 0, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, activation);
 }
 
 int cubert_gemm_skinny_f16(void *handle, int M, int N, int K, float alpha, const cubert_half *A, int lda,
-                           const cubert_half *B, int ldb, cubert_half *C, int ldc, const cubert_half *bias) {
+                           const cubert_half *B, int ldb, cubert_half *C, int ldc, const cubert_half *bias,
+                           int activation) {
     BlasContext *ctx = (BlasContext *) handle;
     if (!ctx || !A || !B || !C) return CUBERT_BAD_ARGUMENT;
-    return run_skinny(ctx, 1, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias);
+    if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;
+    return run_skinny(ctx, 1, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, activation);
 }
 
 int cubert_gemm_strided_batch_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha,

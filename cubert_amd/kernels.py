@@ -158,10 +158,10 @@ class Blas(object):
               ldb, float(beta), _ptr(C), ldc, _ptr(bias))
         return C
 
-    def gemm_skinny(self, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias=None):
-        """C = alpha A B (+ bias) with the few-token kernel (N <= 32); None when the problem does not fit it."""
+    def gemm_skinny(self, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias=None, gelu=False):
+        """C = [gelu](alpha A B (+ bias)) with the few-token kernel (N <= 32); None when the problem does not fit."""
         fn = getattr(lib(), "cubert_gemm_skinny_" + _suffix(C))
-        rc = fn(self.handle, M, N, K, float(alpha), _ptr(A), lda, _ptr(B), ldb, _ptr(C), ldc, _ptr(bias))
+        rc = fn(self.handle, M, N, K, float(alpha), _ptr(A), lda, _ptr(B), ldb, _ptr(C), ldc, _ptr(bias), int(gelu))
         if rc == -2:
             return None
         _check(rc, fn.__name__)

@@ -195,13 +195,17 @@ int cubert_gemm_f16(void *handle, int transA, int transB, int M, int N, int K, f
  * are added in a fixed order, so results do not depend on scheduling.  cubert_gemm_* takes this path by
  * itself when the problem fits (CUBERT_GEMM=library in the environment turns that off).  Needs K a multiple
  * of 16 and B 16-byte aligned with ldb a multiple of 16 bytes; anything else returns CUBERT_UNSUPPORTED and
- * launches nothing.  Calls on one handle must not overlap (they share the handle's scratch).
+ * launches nothing (also with CUBERT_GEMM=library or naive in the environment).  activation: 0 = none, 1 = the
+ * erf-form GELU of cubert_bias_gelu applied to the result (Dense + bias + GELU of BertIntermediate in one
+ * launch; reference src/cuBERT/op_att/Transformer.cpp:164-165).  Calls on one handle must not overlap (they share
+ * the handle's scratch).
  * replaces: Dense<T>::compute -> blas_gemm<T> for small batch * seq_length, reference
  * src/cuBERT/op/Dense.cpp:47-57 (bias: Dense.cpp:41-44). */
 int cubert_gemm_skinny_f32(void *handle, int M, int N, int K, float alpha, const float *A, int lda, const float *B,
-                           int ldb, float *C, int ldc, const float *bias);
+                           int ldb, float *C, int ldc, const float *bias, int activation);
 int cubert_gemm_skinny_f16(void *handle, int M, int N, int K, float alpha, const cubert_half *A, int lda,
-                           const cubert_half *B, int ldb, cubert_half *C, int ldc, const cubert_half *bias);
+                           const cubert_half *B, int ldb, cubert_half *C, int ldc, const cubert_half *bias,
+                           int activation);
 
 /* The same over `batch_count` problems at fixed strides (in elements).
  * replaces: blas_gemm_strided_batch<T>, reference src/cuBERT/common.h:82-92. */

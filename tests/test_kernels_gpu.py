@@ -451,6 +451,12 @@ def test_gemm_skinny_against_oracle_sgemm(K, name, M, N, K_):
             assert_close(host(outs[which][0]), want, 2e-5 if name == "f32" else 2e-3,
                          "gemm_skinny %s alpha=%g" % (name, alpha))
     B, dB = Bs[0], dBs[0]
+    # Dense + bias + GELU in one launch against the oracle's GELU of the oracle's GEMM
+    C = torch.zeros((N * M,), dtype=tdt(name), device="cuda")
+    assert blas.gemm_skinny(M, N, K_, 1.0, dA, M, dB, ldb, C, M, bias=dbias, gelu=True) is not None
+    pre = (oracle.sgemm(0, 0, M, N, K_, 1.0, A, M, B, ldb, 0.0, np.zeros(N * M, np.float32), M).reshape(N, M)
+           + bias[None, :])
+    assert_close(host(C), oracle.gelu(pre).ravel(), 2e-5 if name == "f32" else 2e-3, "gemm_skinny + gelu %s" % name)
     # the general entry point takes the same path by itself
     C = torch.zeros((N * M,), dtype=tdt(name), device="cuda")
     blas.gemm(0, 0, M, N, K_, 1.0, dA, M, dB, ldb, 0.0, C, M, bias=dbias)
