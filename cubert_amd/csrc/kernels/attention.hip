@@ -279,6 +279,7 @@ __global__ __launch_bounds__(kBlock) void attention_context_kernel(const T *__re
 // P never moves.  Scores and probabilities are rounded to the storage type at the points where the
 // three-kernel path stores them, which keeps the two paths within summation-order differences of each other.
 constexpr float kMaskedScore = -10000.0f;
+constexpr float kLog2e = 1.4426950408889634f;
 
 template <typename T>
 __device__ __forceinline__ float normalise_prob(float e, float sum, float inv_sum);
@@ -360,13 +361,7 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
         const int row = idx / kVecPerRow, c = idx - row * kVecPerRow;
         store_vec<T, V>(s_k + row * kPitchK + c * V, kreg[u]);
     }
-#pragma unroll
-    for (int u = 0; u < kLoadsV; ++u) {
-        const int idx = threadIdx.x + u * kThreads;
-        const int j = idx % D, grp = idx / D;
-        store_vec<T, V>(s_vt + j * kPitchV + grp * V, vreg[u]);
-    }
-    __syncthreads();
+    __syncthreads();  // K and the mask are in LDS; the V loads are still in flight
 
     // scores^T[key, query]
     v16f32 p[KT];
@@ -408,6 +403,15 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
     sum += __shfl_xor(sum, 32, kWave);
     const float inv = 1.f / sum;
 
+    // V^T goes to LDS only now: its loads had the whole score and softmax phase to arrive
+#pragma unroll
+    for (int u = 0; u < kLoadsV; ++u) {
+        const int idx = threadIdx.x + u * kThreads;
+        const int j = idx % D, grp = idx / D;
+        store_vec<T, V>(s_vt + j * kPitchV + grp * V, vreg[u]);
+    }
+    __syncthreads();
+
     // ctx[query, column]: A slots = this lane's probabilities, B = the same keys of V^T row (column) jt*32 + r
     v16f32 out[kColTiles];
 #pragma unroll
@@ -441,8 +445,8 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
 // updates the query's running maximum m and sum l, rescales the context accumulators by exp(m_old - m_new) and
 // adds exp(s - m_new) V.  The accumulators have queries along registers while m and l live in the lane of the
 // query, so the per-query factors cross lanes through 128 bytes of wavefront-private LDS.  The result is divided
-// by l once at the end (probabilities are not rounded to the storage type one by one as the three-kernel path
-// does; the difference is within the fp16 storage tolerance).
+// by l once at the end (scores and probabilities are not rounded to the storage type one by one as the
+// three-kernel path does; the difference is within the fp16 storage tolerance).
 template <typename T, int D>
 __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restrict__ q, const T *__restrict__ k,
                                                                const T *__restrict__ v, int ld,
@@ -496,7 +500,7 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
         }
     }
     for (int i = threadIdx.x; i < S; i += threads) {
-        s_mask[i] = (mask != nullptr && !mask[(size_t) b * S + i]) ? kMaskedScore : 0.f;
+        s_mask[i] = (mask != nullptr && !mask[(size_t) b * S + i]) ? kMaskedScore * kLog2e : 0.f;
     }
 #pragma unroll
     for (int u = 0; u < kLoads; ++u) {
@@ -512,6 +516,9 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
     }
     __syncthreads();
 
+    // Scores are kept in units of log 2 (t = s * log2 e), so that exp(s - m) is one v_exp_f32 of t - m_t and the
+    // scale 1/sqrt(d) and the change of base are a single multiply-add with the mask.
+    const float scale = alpha * kLog2e;
     float *factor = s_factor + qt * 32;  // private to this wavefront
     float m = -3.402823466e+38f, l = 0.f;
     v16f32 out[kColTiles];
@@ -535,7 +542,7 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
                     const Vec<float, 4> mk = load_vec<float, 4>(s_mask + kt * 32 + g * 8 + hh * 4);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const float sc = to_f32(from_f32<T>(c[g * 4 + e] * alpha)) + mk.v[e];
+                        const float sc = fmaf(c[g * 4 + e], scale, mk.v[e]);
                         c[g * 4 + e] = sc;
                         cm = fmaxf(cm, sc);
                     }
@@ -548,13 +555,13 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
         }
         cm = fmaxf(cm, __shfl_xor(cm, 32, kWave));
         const float m_new = fmaxf(m, cm);
-        const float f = __expf(m - m_new);  // 0 in the first chunk (m = -max float), where out is 0 anyway
+        const float f = __builtin_amdgcn_exp2f(m - m_new);  // 0 in the first chunk (m = -max float); out is 0 there
         float part = 0.f;
 #pragma unroll
         for (int cc = 0; cc < kChunk; ++cc) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                p[cc][i] = __expf(p[cc][i] - m_new);
+                p[cc][i] = __builtin_amdgcn_exp2f(p[cc][i] - m_new);
                 part += p[cc][i];
             }
         }
@@ -563,7 +570,7 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
         m = m_new;
 
         // rescale the accumulators: row i of a lane is query acc_row(i, hh), whose factor is in lane acc_row(i, hh)
-        if (c0 > 0) {
+        if (c0 > 0 && __any(f != 1.f)) {  // wavefront-uniform: skipped when no query's maximum moved
             if (hh == 0) factor[r] = f;
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): LDS operations of one wavefront complete in order
             __builtin_amdgcn_wave_barrier();
