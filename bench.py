@@ -28,18 +28,21 @@ HBM_PEAK_GBS = 8000.0
 # need the profiler, so these are recorded values, not measured by a plain run.
 MEASURED_TRAFFIC = {
     "C1": {
+        "attention_fused": 50675000,
         "embed_ln": 25286438,
         "mask_scale_softmax": 12588575,
         "bias_res_ln": 37627533,
         "bias_gelu": 100321862
     },
     "C3": {
+        "attention_fused": 200310000,
         "embed_ln": 99683567,
         "mask_scale_softmax": 801872210,
         "bias_res_ln": 150175758,
         "bias_gelu": 400874437
     },
     "C4": {
+        "attention_fused": 266970000,
         "embed_ln": 133391970,
         "mask_scale_softmax": 267485530,
         "bias_res_ln": 200172741,
