@@ -3,13 +3,62 @@
 #include <chrono>
 #include <iostream>
 #include <stdexcept>
+#include <string>
 
 namespace cuBERT {
+
+namespace {
+
+// Every tensor the model will read must hold as many elements as the sizes found in the file and the
+// arguments of cuBERT_open imply; the constructors below copy that many elements without looking again.
+// (The reference trusts the file.)  A tensor that is absent is left to the lookup that needs it.
+template <typename T>
+void check_tensor_sizes(const Graph<T> &g, size_t seq_length, size_t num_hidden_layers) {
+    const size_t H = g.hidden_size, I = g.intermediate_size;
+    auto expect = [&](const std::string &name, size_t want, bool at_least = false) {
+        auto it = g.size.find(name);
+        if (it == g.size.end()) return;
+        if (at_least ? it->second < want : it->second != want) {
+            throw std::invalid_argument("model file invalid: " + name + " holds " + std::to_string(it->second) +
+                                        " elements, the model needs " + std::to_string(want));
+        }
+    };
+    if (H == 0) throw std::invalid_argument("model file invalid: no embedding tables");
+    expect("bert/embeddings/word_embeddings", g.vocab_size * H);
+    expect("bert/embeddings/token_type_embeddings", g.type_vocab_size * H);
+    expect("bert/embeddings/position_embeddings", seq_length * H, true);
+    expect("bert/embeddings/LayerNorm/beta", H);
+    expect("bert/embeddings/LayerNorm/gamma", H);
+    for (size_t l = 0; l < num_hidden_layers; ++l) {
+        const std::string p = "bert/encoder/layer_" + std::to_string(l);
+        for (const char *n : {"query", "key", "value"}) {
+            expect(p + "/attention/self/" + n + "/kernel", H * H);
+            expect(p + "/attention/self/" + n + "/bias", H);
+        }
+        expect(p + "/attention/output/dense/kernel", H * H);
+        expect(p + "/attention/output/dense/bias", H);
+        expect(p + "/attention/output/LayerNorm/beta", H);
+        expect(p + "/attention/output/LayerNorm/gamma", H);
+        expect(p + "/intermediate/dense/kernel", H * I);
+        expect(p + "/intermediate/dense/bias", I);
+        expect(p + "/output/dense/kernel", I * H);
+        expect(p + "/output/dense/bias", H);
+        expect(p + "/output/LayerNorm/beta", H);
+        expect(p + "/output/LayerNorm/gamma", H);
+    }
+    expect("bert/pooler/dense/kernel", H * H);
+    expect("bert/pooler/dense/bias", H);
+    expect("output_weights", g.num_labels * H);
+    expect("output_bias", g.num_labels);
+}
+
+}  // namespace
 
 template <typename T>
 BertM<T>::BertM(const char *model_file, size_t max_batch_size, size_t seq_length, size_t num_hidden_layers,
                 size_t num_attention_heads)
         : seq_length(seq_length), graph(model_file), rr(0) {
+    check_tensor_sizes(graph, seq_length, num_hidden_layers);
     const int count = cuBERT::get_gpu_count();
     if (count == 0) {
         throw std::invalid_argument("No GPU device detected");

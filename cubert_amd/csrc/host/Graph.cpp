@@ -165,7 +165,21 @@ Graph<T>::Graph(const char *filename) {
         else if (value.dtype == kDtHalf) len = (size_t) (value.content.end - value.content.p) / sizeof(half);
         else continue;
 
-        T *data = new T[len];
+        // a declared shape must describe the bytes that are there (a scalar has no dims)
+        unsigned long long declared = 1;
+        for (long long d : value.dims) {
+            if (d < 0 || (d > 0 && declared > (1ull << 40) / (unsigned long long) d)) {
+                throw std::invalid_argument("model file invalid: bad shape of " + name);
+            }
+            declared *= (unsigned long long) d;
+        }
+        if (declared != len) {
+            throw std::invalid_argument("model file invalid: " + name + " holds " + std::to_string(len) +
+                                        " elements, its shape says " + std::to_string(declared));
+        }
+
+        storage.emplace_back(new T[len]);
+        T *data = storage.back().get();
         // tensor_content sits at an arbitrary byte offset of the file: copy out before converting
         if (value.dtype == kDtFloat) {
             std::vector<float> tmp(len);
@@ -176,10 +190,9 @@ Graph<T>::Graph(const char *filename) {
             std::memcpy(tmp.data(), value.content.p, len * sizeof(half));
             T2T(tmp.data(), data, len);
         }
-        auto old = var.find(name);
-        if (old != var.end()) delete[] old->second;
-        var[name] = data;
+        var[name] = data;  // a repeated name keeps its last tensor
         shape[name] = value.dims;
+        this->size[name] = len;
 
         const std::vector<long long> &d = value.dims;
         if (name == "bert/embeddings/word_embeddings" && d.size() >= 2) {
@@ -204,9 +217,7 @@ Graph<T>::Graph(const char *filename) {
 }
 
 template <typename T>
-Graph<T>::~Graph() {
-    for (auto &kv : var) delete[] kv.second;
-}
+Graph<T>::~Graph() = default;
 
 template class Graph<float>;
 template class Graph<half>;

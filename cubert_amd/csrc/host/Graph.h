@@ -11,6 +11,7 @@
 #define CUBERT_HOST_GRAPH_H
 
 #include <cstddef>
+#include <memory>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -30,11 +31,18 @@ public:
 
     std::unordered_map<std::string, T *> var;
     std::unordered_map<std::string, std::vector<long long>> shape;
+    std::unordered_map<std::string, size_t> size;  // elements held by var[name]
+
     size_t vocab_size = 0;
     size_t type_vocab_size = 0;
     size_t hidden_size = 0;
     size_t intermediate_size = 0;
     size_t num_labels = 1;
+
+private:
+    // Owns what var points at.  A member (not the destructor) so that a constructor that throws half way
+    // through a damaged file releases what it had already converted.
+    std::vector<std::unique_ptr<T[]>> storage;
 };
 
 }  // namespace cuBERT

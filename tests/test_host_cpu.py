@@ -126,3 +126,35 @@ def test_generators_are_deterministic_and_follow_the_configs():
     _, mask4, seg4 = config_inputs("C4")
     assert mask4.all() and (seg4[:, 0] == 0).all() and (seg4[:, -1] == 1).all()
     assert set(CONFIGS) == {"C0", "C1", "C2", "C3", "C4"}
+
+
+def test_open_rejects_files_whose_tensors_do_not_fit_the_model(tmp_path):
+    """cuBERT_open checks every tensor's element count against the sizes in the file and its own arguments before
+    anything is copied (the reference trusts the file); this happens before the GPU is looked for, so it runs
+    here.  A consistent file gets as far as the device count."""
+    import cubert_amd
+    from cubert_amd.graphdef import write_graphdef
+    from cubert_amd.testing import random_bert_weights
+    small = dict(vocab=50, hidden=32, layers=2, heads=4, intermediate=64, max_position=16, type_vocab=2)
+    w = random_bert_weights(seed=1, labels=2, **small)
+
+    def open_(weights, seq_length=16, layers=2):
+        path = write_graphdef(str(tmp_path / "m.pb"), weights)
+        model = cubert_amd.Model(path, 2, seq_length, layers, 4)
+        model.close()
+
+    with pytest.raises(ValueError, match="position_embeddings holds 512 elements, the model needs 1024"):
+        open_(w, seq_length=32)                      # longer sequences than the position table has rows
+    bad = dict(w)
+    bad["bert/encoder/layer_1/intermediate/dense/kernel"] = w["bert/encoder/layer_1/intermediate/dense/kernel"][:, :60]
+    with pytest.raises(ValueError, match="layer_1/intermediate/dense/kernel holds 1920 elements, the model needs 2048"):
+        open_(bad)
+    bad = dict(w)
+    bad["output_bias"] = np.zeros(3, np.float32)
+    with pytest.raises(ValueError, match="output_bias holds 3 elements"):
+        open_(bad)
+    if cubert_amd.get_gpu_count() == 0:
+        with pytest.raises(ValueError, match="No GPU device detected"):
+            open_(w)
+    else:
+        open_(w)
