@@ -178,7 +178,7 @@ __global__ __launch_bounds__(kBlock) void ln_pair_kernel(T *__restrict__ inout, 
             src_c[k] = residual + (size_t) (row0 + k) * H;
         }
     }
-    T *dst[2] = {inout + (size_t) row0 * H, inout + (size_t) (row0 + 1) * H};
+    T *dst[1] = {inout + (size_t) row0 * H};
 
     Vec<T, VEC> a[3], b[3], c[3], g[3], be[3];
     int col[3];
@@ -189,10 +189,19 @@ __global__ __launch_bounds__(kBlock) void ln_pair_kernel(T *__restrict__ inout, 
         second[k] = k == 2 || (k == 1 && upper);
         col[k] = second[k] ? flat - H : flat;
         active[k] = !second[k] || has_second;
-        const Vec<T, VEC> zero = {};
-        a[k] = active[k] ? load_vec<T, VEC>((second[k] ? src_a[1] : src_a[0]) + col[k]) : zero;
-        c[k] = active[k] ? load_vec<T, VEC>((second[k] ? src_c[1] : src_c[0]) + col[k]) : zero;
-        if (EMBED) b[k] = active[k] ? load_vec<T, VEC>((second[k] ? src_b[1] : src_b[0]) + col[k]) : zero;
+        // Loads are unconditional (a lane whose row does not exist re-reads the first row and is masked out of
+        // the sums and the stores below), so nothing stands between the loads of a wavefront.
+        if (EMBED) {
+            const bool from_second = second[k] && has_second;
+            a[k] = load_vec<T, VEC>((from_second ? src_a[1] : src_a[0]) + col[k]);
+            c[k] = load_vec<T, VEC>((from_second ? src_c[1] : src_c[0]) + col[k]);
+            b[k] = load_vec<T, VEC>((from_second ? src_b[1] : src_b[0]) + col[k]);
+        } else {
+            // the two rows are adjacent in memory: one base address, the offset inside the two-row span
+            const int at = active[k] ? flat : col[k];
+            a[k] = load_vec<T, VEC>(src_a[0] + at);
+            c[k] = load_vec<T, VEC>(src_c[0] + at);
+        }
     }
 #pragma unroll
     for (int k = 0; k < 3; ++k) {
@@ -200,6 +209,8 @@ __global__ __launch_bounds__(kBlock) void ln_pair_kernel(T *__restrict__ inout, 
         g[k] = load_vec<T, VEC>(gamma + col[k]);
         be[k] = load_vec<T, VEC>(beta + col[k]);
     }
+    // every load above is issued before the first conversion below (loads do not move across this point)
+    asm volatile("" ::: "memory");
     float x[3][VEC], s[3], ss[3];
 #pragma unroll
     for (int k = 0; k < 3; ++k) {
@@ -214,6 +225,10 @@ __global__ __launch_bounds__(kBlock) void ln_pair_kernel(T *__restrict__ inout, 
             s[k] += v;
             ss[k] += v * v;
         }
+        if (!active[k]) {
+            s[k] = 0.f;
+            ss[k] = 0.f;
+        }
     }
     float mean[2], rstd[2];
     ln_stats(s[0] + (upper ? 0.f : s[1]), ss[0] + (upper ? 0.f : ss[1]), H, mean[0], rstd[0]);
@@ -225,7 +240,7 @@ __global__ __launch_bounds__(kBlock) void ln_pair_kernel(T *__restrict__ inout, 
         Vec<T, VEC> o;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) o.v[i] = from_f32<T>(to_f32(be[k].v[i]) + (to_f32(g[k].v[i]) * r) * (x[k][i] - m));
-        if (active[k]) store_vec<T, VEC>((second[k] ? dst[1] : dst[0]) + col[k], o);
+        if (active[k]) store_vec<T, VEC>(dst[0] + (k * kWave + lane) * VEC, o);  // dst rows are adjacent too
     }
 }
 
