@@ -42,6 +42,31 @@ __global__ __launch_bounds__(kBlock) void bias_act_kernel(T *__restrict__ inout,
     }
 }
 
+// The same with the trip count known at compile time (width == TRIPS * blockDim.x * VEC): every load of the
+// thread is issued before the first store, which the in-place loop above cannot do (the compiler must keep a
+// trip's load behind the previous trip's store to the same array).
+template <typename T, typename Op, int VEC, int TRIPS>
+__global__ __launch_bounds__(kBlock) void bias_act_unrolled_kernel(T *__restrict__ inout, const T *__restrict__ bias,
+                                                                   int width) {
+    T *row = inout + (size_t) blockIdx.x * width;
+    Op op;
+    Vec<T, VEC> x[TRIPS], bv[TRIPS];
+#pragma unroll
+    for (int t = 0; t < TRIPS; ++t) x[t] = load_vec<T, VEC>(row + (t * blockDim.x + threadIdx.x) * VEC);
+#pragma unroll
+    for (int t = 0; t < TRIPS; ++t) {
+        bv[t] = Vec<T, VEC>{};
+        if (bias != nullptr) bv[t] = load_vec<T, VEC>(bias + (t * blockDim.x + threadIdx.x) * VEC);
+    }
+#pragma unroll
+    for (int t = 0; t < TRIPS; ++t) {
+        Vec<T, VEC> y;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) y.v[i] = from_f32<T>(op(to_f32(x[t].v[i]) + to_f32(bv[t].v[i])));
+        store_vec<T, VEC>(row + (t * blockDim.x + threadIdx.x) * VEC, y);
+    }
+}
+
 // Threads per workgroup so that the column walk has no ragged last trip when possible.
 inline int pick_threads(int vectors_per_row) {
     for (int t = kBlock; t >= kWave; t -= kWave) {
@@ -57,7 +82,13 @@ int bias_act(T *inout, const T *bias, int rows, int width, void *stream) {
     hipStream_t s = (hipStream_t) stream;
     constexpr int V = MaxVec<T>::value;
     if (width % V == 0 && is_aligned(inout, 16) && (bias == nullptr || is_aligned(bias, 16))) {
-        return launch(bias_act_kernel<T, Op, V>, dim3(rows), dim3(pick_threads(width / V)), s, inout, bias, width);
+        const int threads = pick_threads(width / V);
+        // measured inside the forward pass: fp32 rows of three trips gain 4 % from the unrolled form (batch 128,
+        // seq 32: 17.3 -> 16.6 us); fp16 rows of two trips lose 3-7 % with it, so they keep the loop
+        if (sizeof(T) == 4 && width == threads * V * 3) {
+            return launch(bias_act_unrolled_kernel<T, Op, V, 3>, dim3(rows), dim3(threads), s, inout, bias, width);
+        }
+        return launch(bias_act_kernel<T, Op, V>, dim3(rows), dim3(threads), s, inout, bias, width);
     }
     return launch(bias_act_kernel<T, Op, 1>, dim3(rows), dim3(kBlock), s, inout, bias, width);
 }
