@@ -93,13 +93,15 @@ int bias_act(T *inout, const T *bias, int rows, int width, void *stream) {
     return launch(bias_act_kernel<T, Op, 1>, dim3(rows), dim3(kBlock), s, inout, bias, width);
 }
 
-// out[b, c] = mean_s in[b, s, c].  grid = (column tiles, batch); the block's
-// wavefronts split the sequence, each lane keeps VEC channel sums, and the
-// partial sums meet in LDS.
-template <typename T, int VEC>
-__global__ __launch_bounds__(kBlock) void mean_pool_kernel(const T *__restrict__ in, T *__restrict__ out, int seq,
-                                                           int hidden) {
-    __shared__ float partial[kBlock / kWave][kWave * VEC];
+// out[b, c] = mean_s in[b, s, c].  grid = (column tiles, batch); the block's WAVES wavefronts split the
+// sequence (each keeps four loads in flight), each lane keeps VEC channel sums, and the partial sums meet in
+// LDS in wavefront order.  The launcher picks 8-byte vectors and 16 wavefronts for long sequences so that
+// even a small batch puts a few hundred wavefronts on the chip (batch 32, seq 128, hidden 768: 96 workgroups
+// of 16 wavefronts instead of 64 of 4).
+template <typename T, int VEC, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void mean_pool_kernel(const T *__restrict__ in, T *__restrict__ out,
+                                                                  int seq, int hidden) {
+    __shared__ float partial[WAVES][kWave * VEC];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = wave_in_block();
     const int col = (blockIdx.x * kWave + lane) * VEC;
@@ -109,7 +111,18 @@ __global__ __launch_bounds__(kBlock) void mean_pool_kernel(const T *__restrict__
     for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
     if (col < hidden) {
         const T *p = in + (size_t) b * seq * hidden + col;
-        for (int s = wave; s < seq; s += kBlock / kWave) {
+        int s = wave;
+        for (; s + 3 * WAVES < seq; s += 4 * WAVES) {
+            Vec<T, VEC> v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = load_vec<T, VEC>(p + (size_t) (s + u * WAVES) * hidden);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc[i] += to_f32(v[u].v[i]);
+            }
+        }
+        for (; s < seq; s += WAVES) {
             Vec<T, VEC> v = load_vec<T, VEC>(p + (size_t) s * hidden);
 #pragma unroll
             for (int i = 0; i < VEC; ++i) acc[i] += to_f32(v.v[i]);
@@ -124,7 +137,7 @@ __global__ __launch_bounds__(kBlock) void mean_pool_kernel(const T *__restrict__
         for (int i = 0; i < VEC; ++i) {
             float t = partial[0][lane * VEC + i];
 #pragma unroll
-            for (int w = 1; w < kBlock / kWave; ++w) t += partial[w][lane * VEC + i];
+            for (int w = 1; w < WAVES; ++w) t += partial[w][lane * VEC + i];
             o.v[i] = from_f32<T>(t / (float) seq);
         }
         store_vec<T, VEC>(out + (size_t) b * hidden + col, o);
@@ -136,13 +149,14 @@ int mean_pool(const T *in, T *out, int batch, int seq, int hidden, void *stream)
     if (batch < 0 || seq <= 0 || hidden <= 0 || !in || !out || batch > 65535) return CUBERT_BAD_ARGUMENT;
     if (batch == 0) return 0;
     hipStream_t s = (hipStream_t) stream;
-    constexpr int V = MaxVec<T>::value;
+    constexpr int V = MaxVec<T>::value / 2;  // 8-byte vectors: twice the column tiles of 16-byte ones
     if (hidden % V == 0 && is_aligned(in, 16) && is_aligned(out, 16)) {
         dim3 grid((hidden / V + kWave - 1) / kWave, batch);
-        return launch(mean_pool_kernel<T, V>, grid, dim3(kBlock), s, in, out, seq, hidden);
+        if (seq >= 64) return launch(mean_pool_kernel<T, V, 16>, grid, dim3(16 * kWave), s, in, out, seq, hidden);
+        return launch(mean_pool_kernel<T, V, 4>, grid, dim3(4 * kWave), s, in, out, seq, hidden);
     }
     dim3 grid((hidden + kWave - 1) / kWave, batch);
-    return launch(mean_pool_kernel<T, 1>, grid, dim3(kBlock), s, in, out, seq, hidden);
+    return launch(mean_pool_kernel<T, 1, 4>, grid, dim3(4 * kWave), s, in, out, seq, hidden);
 }
 
 // out[i, :] = table[ids[i], :]; one wavefront per row.
