@@ -21,6 +21,7 @@
 //     transposed in LDS once per workgroup ([head_size][seq + pad]) because an MFMA B operand needs
 //     consecutive k for a fixed column and V is stored with consecutive columns.
 
+#include <atomic>
 #include <initializer_list>
 
 #include "cubert_kernels.h"
@@ -276,8 +277,9 @@ __global__ __launch_bounds__(kBlock) void attention_context_kernel(const T *__re
 // with lane r + 32.  The lane's probabilities are then exactly the A operand slots of the second contraction:
 // a reduction slot may be any key as long as the B operand names the same key, so V is staged transposed
 // ([head column][key]) with the keys permuted into slot order and a lane's B operand is one 16-byte LDS read.
-// P never moves.  Scores and probabilities are rounded to the storage type at the points where the
-// three-kernel path stores them, which keeps the two paths within summation-order differences of each other.
+// P never moves.  Scores stay in fp32 (the three-kernel path rounds them to the storage type when it stores
+// them; the difference is within the fp16 storage tolerance), probabilities are rounded to the storage type as
+// the matrix-core operand they are.
 constexpr float kMaskedScore = -10000.0f;
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -353,7 +355,7 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
         }
     }
     for (int i = threadIdx.x; i < S; i += kThreads) {
-        s_mask[i] = (mask != nullptr && !mask[(size_t) b * S + i]) ? kMaskedScore : 0.f;
+        s_mask[i] = (mask != nullptr && !mask[(size_t) b * S + i]) ? kMaskedScore * kLog2e : 0.f;
     }
 #pragma unroll
     for (int u = 0; u < kLoadsK; ++u) {
@@ -375,7 +377,9 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
         p[kt] = c;
     }
 
-    // register i of tile kt: key kt*32 + acc_row(i, hh), query qt*32 + r
+    // register i of tile kt: key kt*32 + acc_row(i, hh), query qt*32 + r.  Scores are kept in units of log 2
+    // (t = s * log2 e): scale, change of base and mask are one multiply-add, exp(s - max) one v_exp_f32.
+    const float scale = alpha * kLog2e;
     float mx = -3.402823466e+38f;
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
@@ -384,7 +388,7 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
             const Vec<float, 4> m = load_vec<float, 4>(s_mask + kt * 32 + g * 8 + hh * 4);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const float sc = to_f32(from_f32<T>(p[kt][g * 4 + e] * alpha)) + m.v[e];
+                const float sc = fmaf(p[kt][g * 4 + e], scale, m.v[e]);
                 p[kt][g * 4 + e] = sc;
                 mx = fmaxf(mx, sc);
             }
@@ -396,7 +400,7 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
     for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            p[kt][i] = __expf(p[kt][i] - mx);
+            p[kt][i] = __builtin_amdgcn_exp2f(p[kt][i] - mx);
             sum += p[kt][i];
         }
     }
@@ -634,6 +638,23 @@ bool shapes_ok(int batch, int heads, int seq, int head_size, int ld, std::initia
     return true;
 }
 
+// Kernels that ask for more than 48 KB of dynamic LDS need their limit raised once per device (the attribute
+// belongs to the function on the current device).  One bit per device ordinal, set after a successful call.
+template <typename Kernel>
+bool allow_large_lds(Kernel kernel, std::atomic<unsigned long long> &done) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return false;
+    const unsigned long long bit = 1ull << device;
+    if (done.load(std::memory_order_acquire) & bit) return true;
+    if (hipFuncSetAttribute((const void *) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) !=
+        hipSuccess) {
+        (void) hipGetLastError();
+        return false;
+    }
+    done.fetch_or(bit, std::memory_order_release);
+    return true;
+}
+
 template <typename T, int D>
 int launch_scores(const T *q, const T *k, int ld, T *scores, float alpha, int batch, int heads, int seq,
                   hipStream_t s) {
@@ -679,15 +700,8 @@ int launch_context(const T *probs, const T *v, int ld, T *ctx, int ld_ctx, int b
     if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
     auto kernel = attention_context_kernel<T, D>;
     if (lds > 48 * 1024) {
-        static thread_local bool raised = false;  // per instantiation and thread; the call is cheap and idempotent
-        if (!raised) {
-            if (hipFuncSetAttribute((const void *) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) !=
-                hipSuccess) {
-                (void) hipGetLastError();
-                return CUBERT_UNSUPPORTED;
-            }
-            raised = true;
-        }
+        static std::atomic<unsigned long long> raised{0};  // per instantiation
+        if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
     }
     dim3 grid((q_tiles + per_block - 1) / per_block, batch * heads), block(waves * kWave);
     return launch_lds(kernel, grid, block, (unsigned) lds, s, probs, v, ld, ctx, ld_ctx, seq, heads, per_block);
@@ -714,15 +728,8 @@ int launch_fused_kt(const T *q, const T *k, const T *v, int ld, const int8_t *ma
     if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
     auto kernel = attention_fused_kernel<T, D, KT>;
     if (lds > 48 * 1024) {
-        static thread_local bool raised = false;  // per instantiation and thread; the call is cheap and idempotent
-        if (!raised) {
-            if (hipFuncSetAttribute((const void *) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) !=
-                hipSuccess) {
-                (void) hipGetLastError();
-                return CUBERT_UNSUPPORTED;
-            }
-            raised = true;
-        }
+        static std::atomic<unsigned long long> raised{0};  // per instantiation
+        if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
     }
     return launch_untimed(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask, ctx,
                           ld_ctx, alpha, heads);
@@ -749,15 +756,8 @@ int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask,
                        2 * (size_t) seq * sizeof(float);
     if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
     auto kernel = attention_flash_kernel<T, D>;
-    static thread_local bool raised = false;  // per instantiation and thread; the call is cheap and idempotent
-    if (!raised) {
-        if (hipFuncSetAttribute((const void *) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) !=
-            hipSuccess) {
-            (void) hipGetLastError();
-            return CUBERT_UNSUPPORTED;
-        }
-        raised = true;
-    }
+    static std::atomic<unsigned long long> raised{0};  // per instantiation
+    if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
     return launch_untimed(kernel, dim3(batch * heads), dim3(seq / 32 * kWave), (unsigned) lds, s, q, k, v, ld, mask,
                           ctx, ld_ctx, alpha, heads, seq);
 }

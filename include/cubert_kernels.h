@@ -109,11 +109,11 @@ int cubert_attention_context_f16(const cubert_half *probs, const cubert_half *v,
 
 /* The attention core of one layer in a single launch:
  *   ctx[b, q, a, :] = sum_k softmax_k(alpha * Q[b,q,a,:] . K[b,k,a,:] + (mask[b,k] == 0 ? -10000 : 0)) * V[b, k, a, :]
- * with the [batch, heads, seq, seq] scores held in registers (never written to memory).  Up to seq_length 128
- * scores and probabilities are rounded to the storage type where the three-kernel sequence
- * (cubert_attention_scores, cubert_mask_scale_softmax, cubert_attention_context) stores them, so both give the
- * same result up to summation order; from 129 to 512 the softmax runs online over chunks of 64 keys and is
- * normalised once at the end.  mask may be NULL.  Shape support as the two contractions, and seq_length <= 512
+ * with the [batch, heads, seq, seq] scores held in registers in fp32 (never written to memory, never rounded to
+ * the storage type as the three-kernel sequence cubert_attention_scores, cubert_mask_scale_softmax,
+ * cubert_attention_context does; fp32 storage gives the same result up to summation order, fp16 storage agrees
+ * within its tolerance).  Up to seq_length 128 the softmax is the exact two-pass one; from 129 to 512 it runs
+ * online over chunks of 64 keys and is normalised once at the end.  mask may be NULL.  Shape support as the two contractions, and seq_length <= 512
  * (<= 128 for head_size 128, and K, V of one head must fit 160 KB of LDS: fp32 up to seq_length 256 at head size
  * 64); anything else returns CUBERT_UNSUPPORTED and launches nothing.
  * replaces: AttentionSelf<T>::_in_compute's Att_Q_K -> Softmax -> Att_QK_V sequence and the mask tensor of
