@@ -82,6 +82,7 @@ SIGNATURES = {
     "cubert_event_record": (ci, [vp, vp]),
     "cubert_event_elapsed_ms": (ci, [vp, vp, ctypes.POINTER(cf)]),
     "cubert_time_next_launch": (ci, [vp, vp]),
+    "cubert_gemm_skinny_packed_elements": (ctypes.c_size_t, [ci, ci]),
     "cubert_blas_create": (vp, []),
     "cubert_blas_destroy": (ci, [vp]),
     "cubert_blas_set_stream": (ci, [vp, vp]),
@@ -103,6 +104,8 @@ for _t in ("f32", "f16"):
         "cubert_mean_pool_" + _t: (ci, [vp, vp, ci, ci, ci, vp]),
         "cubert_gemm_" + _t: (ci, [vp, ci, ci, ci, ci, ci, cf, vp, ci, vp, ci, cf, vp, ci, vp]),
         "cubert_gemm_skinny_" + _t: (ci, [vp, ci, ci, ci, cf, vp, ci, vp, ci, vp, ci, vp, ci]),
+        "cubert_gemm_skinny_pack_" + _t: (ci, [vp, vp, ci, ci, ci, vp]),
+        "cubert_gemm_skinny_packed_" + _t: (ci, [vp, ci, ci, ci, cf, vp, vp, ci, vp, ci, vp, ci]),
         "cubert_gemm_strided_batch_" + _t: (ci, [vp, ci, ci, ci, ci, ci, cf, vp, ci, cll, vp, ci, cll, cf, vp, ci, cll, ci]),
     })
 

@@ -3,16 +3,18 @@
 // named-weight map under a variable prefix, then compute(batch, input, mask)
 // with device pointers, returning a device pointer to [batch, seq, hidden].
 //
-// Inside, a layer is 6 GEMMs and 3 fused kernels:
+// Inside, a layer is 8 launches (7 for at most 32 tokens):
 //   qkv   = x * [Wq|Wk|Wv] + [bq|bk|bv]          one GEMM, bias in its epilogue
-//   s     = (1/sqrt d) * Q K^T                    batched GEMM into scores[B, A, S, S]
-//   p     = softmax(s + mask)                     mask_scale_softmax_      (fused kernel)
-//   ctx   = p V                                   batched GEMM
+//   ctx   = softmax((1/sqrt d) Q K^T + mask) V    one attention kernel (scores stay in registers); where its
+//                                                 shape limits do not hold: scores kernel or batched GEMM into
+//                                                 scores[B, A, S, S], mask_scale_softmax_, context kernel or GEMM
 //   a     = LN(ctx * Wo + bo + x)                 GEMM, then layer_norm_   (fused kernel)
-//   i     = GELU(a * Wi + bi)                     GEMM, then gelu          (fused kernel)
+//   i     = GELU(a * Wi + bi)                     GEMM, then gelu          (fused kernel; one launch for both at
+//                                                 <= 32 tokens)
 //   out   = LN(i * Wout + bout + a)               GEMM, then layer_norm_   (fused kernel)
 // Activation buffers are shared by all layers (the reference keeps four private
-// buffers per layer); weights live in one device allocation.
+// buffers per layer); weights live in one device allocation.  A half-precision model whose seq_length allows
+// requests of at most 32 tokens also keeps its four Dense kernels in the few-token GEMM kernel's own order.
 #ifndef CUBERT_HOST_TRANSFORMER_H
 #define CUBERT_HOST_TRANSFORMER_H
 
@@ -56,15 +58,23 @@ private:
         T *intermediate_kernel, *intermediate_bias;
         T *output_kernel, *output_bias;
         T *output_norm_beta, *output_norm_gamma;
+        // the Dense kernels again, in the few-token GEMM kernel's order (null when not kept)
+        T *qkv_packed = nullptr, *attention_output_packed = nullptr, *intermediate_packed = nullptr,
+          *output_packed = nullptr;
     };
 
     void layout_weights();
     void layout_buffers();
     void attention(size_t batch_size, const T *qkv, const int8_t *mask);
+    // out[tokens, out_features] = in[tokens, in_features] * kernel (+ bias) (, GELU); returns whether bias and
+    // activation were applied (false: the caller's fused kernel still has to).
+    bool dense(int out_features, int tokens, int in_features, const T *kernel, const T *packed, const T *in, T *out,
+               const T *bias, bool bias_in_gemm, bool gelu);
 
     void *cublas;
     Profiler *profiler = nullptr;
     bool dense_gelu_fits = true;       // cleared when the few-token Dense + GELU kernel declines this model's shape
+    bool keep_packed = false;          // Dense kernels are also kept in the few-token kernel's order
     bool fused_attention_fits = true;  // cleared when the one-launch attention kernel declines this model's shape
     size_t max_batch_size, seq_length, hidden_size, num_hidden_layers, num_attention_heads, intermediate_size;
 

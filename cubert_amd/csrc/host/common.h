@@ -82,21 +82,31 @@ inline void blas_gemm(void *handle, bool TransA, bool TransB, int M, int N, int 
                       const half *B, int ldb, float beta, half *C, int ldc, const half *bias = nullptr) {
     CUBERT_CHECK(cubert_gemm_f16(handle, TransA, TransB, M, N, K, alpha, h(A), lda, h(B), ldb, beta, h(C), ldc, h(bias)));
 }
-// Dense + bias + GELU in one launch for at most 32 tokens (column-major C[M, N] = gelu(A B + bias), N <= 32);
-// false when the few-token kernel does not take the problem (the caller then runs blas_gemm and gelu).
-inline bool dense_gelu_few_tokens(void *handle, int M, int N, int K, const float *A, int lda, const float *B, int ldb,
-                                  float *C, int ldc, const float *bias) {
-    const int rc = cubert_gemm_skinny_f32(handle, M, N, K, 1.f, A, lda, B, ldb, C, ldc, bias, 1);
+// A Dense layer for at most 32 tokens on the few-token kernel (column-major C[M, N] = [gelu](A B + bias), N <= 32),
+// on the weights in its own order when `packed` is given; false when the kernel does not take the problem
+// (the caller then runs blas_gemm).  No counterpart in the reference.
+inline bool dense_few_tokens(void *handle, int M, int N, int K, const float *A, int lda, const float *packed,
+                             const float *B, int ldb, float *C, int ldc, const float *bias, bool gelu) {
+    const int rc = packed ? cubert_gemm_skinny_packed_f32(handle, M, N, K, 1.f, packed, B, ldb, C, ldc, bias, gelu)
+                          : cubert_gemm_skinny_f32(handle, M, N, K, 1.f, A, lda, B, ldb, C, ldc, bias, gelu);
     if (rc == CUBERT_UNSUPPORTED) return false;
     CUBERT_CHECK(rc);
     return true;
 }
-inline bool dense_gelu_few_tokens(void *handle, int M, int N, int K, const half *A, int lda, const half *B, int ldb,
-                                  half *C, int ldc, const half *bias) {
-    const int rc = cubert_gemm_skinny_f16(handle, M, N, K, 1.f, h(A), lda, h(B), ldb, h(C), ldc, h(bias), 1);
+inline bool dense_few_tokens(void *handle, int M, int N, int K, const half *A, int lda, const half *packed,
+                             const half *B, int ldb, half *C, int ldc, const half *bias, bool gelu) {
+    const int rc = packed ? cubert_gemm_skinny_packed_f16(handle, M, N, K, 1.f, h(packed), h(B), ldb, h(C), ldc, h(bias),
+                                                          gelu)
+                          : cubert_gemm_skinny_f16(handle, M, N, K, 1.f, h(A), lda, h(B), ldb, h(C), ldc, h(bias), gelu);
     if (rc == CUBERT_UNSUPPORTED) return false;
     CUBERT_CHECK(rc);
     return true;
+}
+inline void pack_few_token_weights(void *handle, const float *A, int lda, int M, int K, float *packed) {
+    CUBERT_CHECK(cubert_gemm_skinny_pack_f32(handle, A, lda, M, K, packed));
+}
+inline void pack_few_token_weights(void *handle, const half *A, int lda, int M, int K, half *packed) {
+    CUBERT_CHECK(cubert_gemm_skinny_pack_f16(handle, h(A), lda, M, K, h(packed)));
 }
 
 inline void blas_gemm_strided_batch(void *handle, bool TransA, bool TransB, int m, int n, int k, float alpha,

@@ -31,7 +31,24 @@ constexpr int kSkinnyChunk = 16;  // reduction values a wavefront consumes per p
 // Accumulator register i of the lane half hh holds this row of a 32x32 MFMA result (column = lane % 32).
 __device__ __forceinline__ int acc_row(int i, int hh) { return (i >> 2) * 8 + hh * 4 + (i & 3); }
 
-template <typename T, bool GELU>
+// Weights in the order the kernel consumes them: for feature block fb and chunk c (16 reduction values), lane
+// (r, hh) finds its 8 operand values A[c*16 + hh*8 + t, fb*32 + r], t < 8, in 8 consecutive elements, so a
+// workgroup's slice of the weights is one contiguous run (32 KB for fp32) read with 16-byte loads instead of
+// 128-byte pieces at a stride of a weight row.  Features past M are stored as zeros.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void gemm_skinny_pack_kernel(const T *__restrict__ A, int lda, int M, int chunks,
+                                                                  T *__restrict__ packed, size_t total) {
+    const size_t idx = (size_t) blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= total) return;
+    const int t = (int) (idx % 8), lane = (int) ((idx / 8) % kWave);
+    const size_t tile = idx / (8 * kWave);
+    const int c = (int) (tile % chunks), fb = (int) (tile / chunks);
+    const int r = lane & 31, hh = lane >> 5;
+    const int k = c * kSkinnyChunk + hh * 8 + t, feature = fb * 32 + r;
+    packed[idx] = feature < M ? A[(size_t) k * lda + feature] : from_f32<T>(0.f);
+}
+
+template <typename T, bool GELU, bool PACKED>
 __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__restrict__ A, int lda,
                                                                      const T *__restrict__ B, int ldb,
                                                                      const T *__restrict__ bias, T *__restrict__ C,
@@ -61,8 +78,18 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
 #pragma unroll
             for (int e = 0; e < V; ++e) x[u * V + e] = to_f32(xv.v[e]);
         }
+        if (PACKED) {
+            const T *src = A + (((size_t) blockIdx.x * chunks + c) * kWave + lane) * 8;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) w[t] = feature < M ? to_f32(A[(size_t) (kb + t) * lda + feature]) : 0.f;
+            for (int u = 0; u < 8 / V; ++u) {
+                const Vec<T, V> wv = load_vec<T, V>(src + u * V);
+#pragma unroll
+                for (int e = 0; e < V; ++e) w[u * V + e] = to_f32(wv.v[e]);
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) w[t] = feature < M ? to_f32(A[(size_t) (kb + t) * lda + feature]) : 0.f;
+        }
 #pragma unroll
         for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[t], w[t], acc, 0, 0, 0);
     }
@@ -123,13 +150,15 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
 // Launches the kernel when the problem fits it, else returns CUBERT_UNSUPPORTED and launches nothing.
 // activation: 0 = none, 1 = erf-form GELU applied to alpha * A B + bias (the BertIntermediate layer).
 // `partials` holds partial_floats floats, `counters` n_counters ints that are zero between launches.
+// packed != 0: A is the output of gemm_skinny_pack for the same M and K (lda is ignored).
 template <typename T>
-int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, const T *B, int ldb, T *C, int ldc,
+int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, int packed, const T *B, int ldb, T *C, int ldc,
                 const T *bias, int activation, float *partials, size_t partial_floats, int *counters,
                 int n_counters, hipStream_t stream) {
     if (activation != 0 && activation != 1) return CUBERT_BAD_ARGUMENT;
     if (M <= 0 || N <= 0 || N > 32 || K <= 0 || K % kSkinnyChunk != 0) return CUBERT_UNSUPPORTED;
-    if (lda < M || ldb < K || ldc < M) return CUBERT_BAD_ARGUMENT;
+    if ((!packed && lda < M) || ldb < K || ldc < M) return CUBERT_BAD_ARGUMENT;
+    if (packed && !is_aligned(A, 16)) return CUBERT_BAD_ARGUMENT;
     if (!is_aligned(B, 16) || (ldb * sizeof(T)) % 16 != 0) return CUBERT_UNSUPPORTED;
     const int blocks = (M + 31) / 32;
     const int chunks = K / kSkinnyChunk;
@@ -142,17 +171,37 @@ int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, const T *
     }
     if (blocks > 65535 || slices > 65535 || (slices > 1 && blocks > n_counters)) return CUBERT_UNSUPPORTED;
     const dim3 grid(blocks, slices), block(kSkinnyThreads);
+#define CUBERT_SKINNY_LAUNCH(GELU, PACKED)                                                                         \
+    return launch(gemm_skinny_kernel<T, GELU, PACKED>, grid, block, stream, A, lda, B, ldb, bias, C, ldc, M, N, K, \
+                  alpha, partials, counters, chunks_per_slice)
     if (activation == 1) {
-        return launch(gemm_skinny_kernel<T, true>, grid, block, stream, A, lda, B, ldb, bias, C, ldc, M, N, K, alpha,
-                      partials, counters, chunks_per_slice);
+        if (packed) CUBERT_SKINNY_LAUNCH(true, true);
+        CUBERT_SKINNY_LAUNCH(true, false);
     }
-    return launch(gemm_skinny_kernel<T, false>, grid, block, stream, A, lda, B, ldb, bias, C, ldc, M, N, K, alpha,
-                  partials, counters, chunks_per_slice);
+    if (packed) CUBERT_SKINNY_LAUNCH(false, true);
+    CUBERT_SKINNY_LAUNCH(false, false);
+#undef CUBERT_SKINNY_LAUNCH
 }
 
-template int gemm_skinny<float>(int, int, int, float, const float *, int, const float *, int, float *, int,
+// Elements of the packed form of an [K, M] weight matrix.
+size_t gemm_skinny_packed_elements(int M, int K) { return (size_t) ((M + 31) / 32) * 32 * (size_t) K; }
+
+template <typename T>
+int gemm_skinny_pack(const T *A, int lda, int M, int K, T *packed, hipStream_t stream) {
+    if (!A || !packed || M <= 0 || K <= 0 || lda < M) return CUBERT_BAD_ARGUMENT;
+    if (K % kSkinnyChunk != 0 || !is_aligned(packed, 16)) return CUBERT_UNSUPPORTED;
+    const size_t total = gemm_skinny_packed_elements(M, K);
+    const size_t blocks = (total + kBlock - 1) / kBlock;
+    if (blocks > 0x7fffffffull) return CUBERT_UNSUPPORTED;
+    return launch(gemm_skinny_pack_kernel<T>, dim3((unsigned) blocks), dim3(kBlock), stream, A, lda, M,
+                  K / kSkinnyChunk, packed, total);
+}
+
+template int gemm_skinny<float>(int, int, int, float, const float *, int, int, const float *, int, float *, int,
                                 const float *, int, float *, size_t, int *, int, hipStream_t);
-template int gemm_skinny<half_t>(int, int, int, float, const half_t *, int, const half_t *, int, half_t *, int,
+template int gemm_skinny<half_t>(int, int, int, float, const half_t *, int, int, const half_t *, int, half_t *, int,
                                  const half_t *, int, float *, size_t, int *, int, hipStream_t);
+template int gemm_skinny_pack<float>(const float *, int, int, int, float *, hipStream_t);
+template int gemm_skinny_pack<half_t>(const half_t *, int, int, int, half_t *, hipStream_t);
 
 }  // namespace cubert

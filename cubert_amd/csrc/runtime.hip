@@ -24,9 +24,12 @@
 namespace cubert {
 // kernels/gemm_skinny.hip
 template <typename T>
-int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, const T *B, int ldb, T *C, int ldc,
+int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, int packed, const T *B, int ldb, T *C, int ldc,
                 const T *bias, int activation, float *partials, size_t partial_floats, int *counters,
                 int n_counters, hipStream_t stream);
+size_t gemm_skinny_packed_elements(int M, int K);
+template <typename T>
+int gemm_skinny_pack(const T *A, int lda, int M, int K, T *packed, hipStream_t stream);
 
 LaunchTiming &pending_launch_timing() {
     static thread_local LaunchTiming pending;
@@ -212,13 +215,13 @@ bool library_gemm_only() {
 }
 
 int run_skinny(BlasContext *ctx, int type, int M, int N, int K, float alpha, const void *A, int lda, const void *B,
-               int ldb, void *C, int ldc, const void *bias, int activation) {
+               int ldb, void *C, int ldc, const void *bias, int activation, int packed = 0) {
     if (type == 0) {
-        return cubert::gemm_skinny<float>(M, N, K, alpha, (const float *) A, lda, (const float *) B, ldb, (float *) C,
+        return cubert::gemm_skinny<float>(M, N, K, alpha, (const float *) A, lda, packed, (const float *) B, ldb, (float *) C,
                                           ldc, (const float *) bias, activation, ctx->skinny_partials,
                                           kSkinnyPartialFloats, ctx->skinny_counters, kSkinnyCounters, ctx->stream);
     }
-    return cubert::gemm_skinny<cubert::half_t>(M, N, K, alpha, (const cubert::half_t *) A, lda,
+    return cubert::gemm_skinny<cubert::half_t>(M, N, K, alpha, (const cubert::half_t *) A, lda, packed,
                                                (const cubert::half_t *) B, ldb, (cubert::half_t *) C, ldc,
                                                (const cubert::half_t *) bias, activation, ctx->skinny_partials,
                                                kSkinnyPartialFloats, ctx->skinny_counters, kSkinnyCounters,
@@ -417,6 +420,38 @@ int cubert_gemm_skinny_f16(void *handle, int M, int N, int K, float alpha, const
     if (!ctx || !A || !B || !C) return CUBERT_BAD_ARGUMENT;
     if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;
     return run_skinny(ctx, 1, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, activation);
+}
+
+size_t cubert_gemm_skinny_packed_elements(int M, int K) { return cubert::gemm_skinny_packed_elements(M, K); }
+
+int cubert_gemm_skinny_pack_f32(void *handle, const float *A, int lda, int M, int K, float *packed) {
+    BlasContext *ctx = (BlasContext *) handle;
+    if (!ctx) return CUBERT_BAD_ARGUMENT;
+    return cubert::gemm_skinny_pack<float>(A, lda, M, K, packed, ctx->stream);
+}
+
+int cubert_gemm_skinny_pack_f16(void *handle, const cubert_half *A, int lda, int M, int K, cubert_half *packed) {
+    BlasContext *ctx = (BlasContext *) handle;
+    if (!ctx) return CUBERT_BAD_ARGUMENT;
+    return cubert::gemm_skinny_pack<cubert::half_t>((const cubert::half_t *) A, lda, M, K, (cubert::half_t *) packed,
+                                                    ctx->stream);
+}
+
+int cubert_gemm_skinny_packed_f32(void *handle, int M, int N, int K, float alpha, const float *packedA, const float *B,
+                                  int ldb, float *C, int ldc, const float *bias, int activation) {
+    BlasContext *ctx = (BlasContext *) handle;
+    if (!ctx || !packedA || !B || !C) return CUBERT_BAD_ARGUMENT;
+    if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;
+    return run_skinny(ctx, 0, M, N, K, alpha, packedA, 0, B, ldb, C, ldc, bias, activation, 1);
+}
+
+int cubert_gemm_skinny_packed_f16(void *handle, int M, int N, int K, float alpha, const cubert_half *packedA,
+                                  const cubert_half *B, int ldb, cubert_half *C, int ldc, const cubert_half *bias,
+                                  int activation) {
+    BlasContext *ctx = (BlasContext *) handle;
+    if (!ctx || !packedA || !B || !C) return CUBERT_BAD_ARGUMENT;
+    if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;
+    return run_skinny(ctx, 1, M, N, K, alpha, packedA, 0, B, ldb, C, ldc, bias, activation, 1);
 }
 
 int cubert_gemm_strided_batch_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha,

@@ -167,6 +167,21 @@ class Blas(object):
         _check(rc, fn.__name__)
         return C
 
+    def gemm_skinny_pack(self, A, lda, M, K):
+        """The weight matrix A (M x K column-major, i.e. [K, M] row-major) in the few-token kernel's own order."""
+        packed = torch.empty(lib().cubert_gemm_skinny_packed_elements(M, K), dtype=A.dtype, device=A.device)
+        fn = getattr(lib(), "cubert_gemm_skinny_pack_" + _suffix(A))
+        _check(fn(self.handle, _ptr(A), lda, M, K, _ptr(packed)), fn.__name__)
+        return packed
+
+    def gemm_skinny_packed(self, M, N, K, alpha, packed, B, ldb, C, ldc, bias=None, gelu=False):
+        fn = getattr(lib(), "cubert_gemm_skinny_packed_" + _suffix(C))
+        rc = fn(self.handle, M, N, K, float(alpha), _ptr(packed), _ptr(B), ldb, _ptr(C), ldc, _ptr(bias), int(gelu))
+        if rc == -2:
+            return None
+        _check(rc, fn.__name__)
+        return C
+
     def gemm_strided_batch(self, transA, transB, M, N, K, alpha, A, lda, sA, B, ldb, sB, beta, C, ldc, sC, batch):
         _call("cubert_gemm_strided_batch", C, self.handle, int(transA), int(transB), M, N, K, float(alpha), _ptr(A),
               lda, sA, _ptr(B), ldb, sB, float(beta), _ptr(C), ldc, sC, batch)

@@ -207,6 +207,21 @@ int cubert_gemm_skinny_f16(void *handle, int M, int N, int K, float alpha, const
                            const cubert_half *B, int ldb, cubert_half *C, int ldc, const cubert_half *bias,
                            int activation);
 
+/* The few-token kernel on weights re-ordered once into the order it consumes them (a workgroup then streams
+ * one contiguous run with 16-byte loads instead of 128-byte pieces at a stride of a weight row).
+ * cubert_gemm_skinny_packed_elements(M, K) elements are needed for the packed copy of an A of M x K;
+ * cubert_gemm_skinny_pack_* fills it (asynchronous, on the handle's stream; K a multiple of 16, packed 16-byte
+ * aligned, else CUBERT_UNSUPPORTED); cubert_gemm_skinny_packed_* is cubert_gemm_skinny_* on the packed copy.
+ * No counterpart in the reference (its weights stay in the TensorFlow layout, src/cuBERT/op/Dense.cpp:14-38). */
+size_t cubert_gemm_skinny_packed_elements(int M, int K);
+int cubert_gemm_skinny_pack_f32(void *handle, const float *A, int lda, int M, int K, float *packed);
+int cubert_gemm_skinny_pack_f16(void *handle, const cubert_half *A, int lda, int M, int K, cubert_half *packed);
+int cubert_gemm_skinny_packed_f32(void *handle, int M, int N, int K, float alpha, const float *packedA, const float *B,
+                                  int ldb, float *C, int ldc, const float *bias, int activation);
+int cubert_gemm_skinny_packed_f16(void *handle, int M, int N, int K, float alpha, const cubert_half *packedA,
+                                  const cubert_half *B, int ldb, cubert_half *C, int ldc, const cubert_half *bias,
+                                  int activation);
+
 /* The same over `batch_count` problems at fixed strides (in elements).
  * replaces: blas_gemm_strided_batch<T>, reference src/cuBERT/common.h:82-92. */
 int cubert_gemm_strided_batch_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha,

@@ -98,6 +98,34 @@ def test_small_model_fp16(cb):
         assert_close(got[k], want[k], FP16_TOL, k)
 
 
+@pytest.mark.parametrize("compute_type", [0, 1])
+@pytest.mark.parametrize("seq_length", [32, 16])
+def test_requests_of_at_most_32_tokens(cb, compute_type, seq_length):
+    """Batch 1 (and batch 2 at seq 16) run the Dense layers on the few-token kernel, the intermediate layer with
+    its GELU in the same launch, and a half-precision model on its re-ordered weight copies; a larger batch of the
+    same model takes the library GEMM.  Both must match the oracle, and the single request must match itself as a
+    row of the larger batch."""
+    from cubert_amd.testing import random_bert_weights, random_inputs
+    w = random_bert_weights(seed=11, labels=2, pooler=True, classifier=True, ln_random=True, **SMALL)
+    ids, mask, seg = random_inputs(seed=12, batch=6, seq_length=seq_length, vocab=SMALL["vocab"], min_valid=3,
+                                   segment_split=7)
+    tol = FP16_TOL if compute_type else FP32_TOL
+    wo = {k: oracle.round_to_half(v) for k, v in w.items()} if compute_type else w
+    want = oracle.bert_forward(wo, ids, mask, seg, 3, 4)
+    bert = cb.Bert(w, 6, seq_length, 3, 4, compute_type)
+    full = bert.forward(ids, mask, seg)
+    for n in (1, 2):
+        if n * seq_length > 32:
+            continue
+        few = bert.forward(ids[:n], mask[:n], seg[:n])
+        for k in ("sequence_output", "pooled_output", "logits", "probs"):
+            assert_close(few[k], want[k][:n], tol, "%s, %d request(s)" % (k, n))
+            assert_close(few[k], full[k][:n], tol, "%s vs the same rows of a batch of 6" % k)
+    bert.close()
+    for k in ("sequence_output", "pooled_output", "logits"):
+        assert_close(full[k], want[k], tol, k)
+
+
 def test_repeated_calls_and_smaller_batches_reuse_buffers(cb):
     """The reference's BertMTest calls one model four times; results must not depend on what ran before."""
     from cubert_amd.testing import random_bert_weights, random_inputs
