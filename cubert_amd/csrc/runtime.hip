@@ -52,6 +52,7 @@ hipMemcpyKind copy_kind(int kind) {
 }
 
 constexpr size_t kWorkspaceBytes = 64u << 20;
+constexpr int kMaxCandidates = 32;
 // scratch of the few-token GEMM kernel: partial tiles (fp32) and one arrival counter per feature block
 constexpr size_t kSkinnyPartialFloats = 1u << 20;
 constexpr int kSkinnyCounters = 4096;
@@ -75,12 +76,16 @@ struct GemmPlan {
     hipblasLtMatmulAlgo_t algo;
     size_t workspace = 0;
     bool ok = false;  // false: hipBLASLt has no algorithm for this shape, the plain kernel runs instead
+    // what the heuristic returned, best first by its own ranking; `algo` is one of them
+    std::vector<hipblasLtMatmulHeuristicResult_t> candidates;
+    bool tuned = false;  // `algo` was chosen by timing (or timing does not apply to this plan)
 };
 
 struct BlasContext {
     hipblasLtHandle_t lt = nullptr;
     hipStream_t stream = nullptr;
     void *workspace = nullptr;
+    hipEvent_t tune_start = nullptr, tune_stop = nullptr;  // created on first use
     float *skinny_partials = nullptr;
     int *skinny_counters = nullptr;  // zero between launches (the kernel resets what it counted)
     std::map<GemmKey, GemmPlan> plans;
@@ -132,10 +137,10 @@ int build_plan(BlasContext *ctx, const GemmKey &k, GemmPlan *plan) {
     LT_TRY(hipblasLtMatmulPreferenceCreate(&pref));
     uint64_t ws = kWorkspaceBytes;
     LT_TRY(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof ws));
-    hipblasLtMatmulHeuristicResult_t found[8];
+    hipblasLtMatmulHeuristicResult_t found[kMaxCandidates];
     int n = 0;
     hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(ctx->lt, plan->desc, plan->a, plan->b, plan->c, plan->c, pref,
-                                                         8, found, &n);
+                                                         kMaxCandidates, found, &n);
     hipblasLtMatmulPreferenceDestroy(pref);
     if (st != HIPBLAS_STATUS_SUCCESS || n == 0) {
         if (getenv("CUBERT_VERBOSE")) {
@@ -149,8 +154,106 @@ int build_plan(BlasContext *ctx, const GemmKey &k, GemmPlan *plan) {
     }
     plan->algo = found[0].algo;
     plan->workspace = found[0].workspaceSize;
+    plan->candidates.assign(found, found + n);
     plan->ok = true;
     return 0;
+}
+
+// ---- choosing among the heuristic's candidates by timing -------------------------------------------------
+// The heuristic ranks algorithms without knowing the data; on this part the matrix cores are power limited and
+// the ranking moves with the operand values (measured on the Dense shapes of batch 128 x seq 32 fp32 and of
+// BERT-large batch 256 x seq 128 fp16 with random operands: its first choice is 7-18 % slower than the best of
+// its 32 candidates).  So the first call of a large enough GEMM shape times every candidate on the caller's
+// own operands (beta = 0 only: the output is simply overwritten each time) and keeps the fastest.  The choice
+// is remembered per shape for the whole process, so that every context computes a shape the same way.
+// CUBERT_GEMM_TUNE=0 in the environment keeps the heuristic's first choice.  (The reference exposes the same
+// decision as its GEMM_ALGO_* environment variables, src/cuBERT/common.cpp:106-160.)
+
+constexpr double kTuneMinFlops = 1e9;
+constexpr int kTuneRuns = 8;
+constexpr float kTuneMinGain = 0.97f;  // leave the heuristic's first choice unless another is at least 3 % faster
+
+bool tuning_enabled() {
+    static const bool on = [] {
+        const char *v = getenv("CUBERT_GEMM_TUNE");
+        return v == nullptr || std::string(v) != "0";
+    }();
+    return on;
+}
+
+std::mutex &tuned_mutex() {
+    static std::mutex m;
+    return m;
+}
+std::map<GemmKey, int> &tuned_ranks() {
+    static std::map<GemmKey, int> ranks;
+    return ranks;
+}
+
+void tune_plan(BlasContext *ctx, const GemmKey &k, GemmPlan &p, float alpha, const void *A, const void *B, void *C) {
+    p.tuned = true;
+    const double flops = 2.0 * k.M * k.N * k.K * k.batch;
+    if (!tuning_enabled() || !k.beta_zero || p.candidates.size() < 2 || flops < kTuneMinFlops) return;
+    {
+        std::lock_guard<std::mutex> lock(tuned_mutex());
+        auto it = tuned_ranks().find(k);
+        if (it != tuned_ranks().end()) {
+            if (it->second < (int) p.candidates.size()) {
+                p.algo = p.candidates[it->second].algo;
+                p.workspace = p.candidates[it->second].workspaceSize;
+            }
+            return;
+        }
+    }
+    if (ctx->tune_start == nullptr) {
+        if (hipEventCreate(&ctx->tune_start) != hipSuccess || hipEventCreate(&ctx->tune_stop) != hipSuccess) {
+            (void) hipGetLastError();
+            return;
+        }
+    }
+    const float beta = 0.f;
+    int best = 0;
+    float best_ms = 0.f, first_ms = 0.f;
+    for (int i = 0; i < (int) p.candidates.size(); ++i) {
+        hipblasLtMatmulAlgo_t *algo = &p.candidates[i].algo;
+        bool ok = hipblasLtMatmul(ctx->lt, p.desc, &alpha, A, p.a, B, p.b, &beta, C, p.c, C, p.c, algo, ctx->workspace,
+                                  kWorkspaceBytes, ctx->stream) == HIPBLAS_STATUS_SUCCESS;  // warm-up, also a check
+        if (!ok) continue;
+        if (hipEventRecord(ctx->tune_start, ctx->stream) != hipSuccess) return;
+        for (int r = 0; r < kTuneRuns && ok; ++r) {
+            ok = hipblasLtMatmul(ctx->lt, p.desc, &alpha, A, p.a, B, p.b, &beta, C, p.c, C, p.c, algo, ctx->workspace,
+                                 kWorkspaceBytes, ctx->stream) == HIPBLAS_STATUS_SUCCESS;
+        }
+        float ms = 0.f;
+        if (hipEventRecord(ctx->tune_stop, ctx->stream) != hipSuccess ||
+            hipEventSynchronize(ctx->tune_stop) != hipSuccess ||
+            hipEventElapsedTime(&ms, ctx->tune_start, ctx->tune_stop) != hipSuccess) {
+            (void) hipGetLastError();
+            return;
+        }
+        if (!ok) continue;
+        if (i == 0) first_ms = ms;
+        if (best_ms == 0.f || ms < best_ms) {
+            best_ms = ms;
+            best = i;
+        }
+    }
+    if (best_ms == 0.f) return;
+    if (first_ms > 0.f && best_ms > kTuneMinGain * first_ms) {  // differences of a few per cent do not survive inside a forward pass
+        best = 0;
+        best_ms = first_ms;
+    }
+    p.algo = p.candidates[best].algo;
+    p.workspace = p.candidates[best].workspaceSize;
+    {
+        std::lock_guard<std::mutex> lock(tuned_mutex());
+        tuned_ranks()[k] = best;
+    }
+    if (getenv("CUBERT_VERBOSE")) {
+        fprintf(stderr, "hipBLASLt: gemm type=%d trans=%d%d M=%d N=%d K=%d batch=%d bias=%d: candidate %d of %d, %.1f us\n",
+                k.type, k.transA, k.transB, k.M, k.N, k.K, k.batch, (int) k.bias, best, (int) p.candidates.size(),
+                best_ms * 1e3 / kTuneRuns);
+    }
 }
 
 // Plain one-thread-per-output GEMM (fp32 accumulation, k ascending).  Used for shapes hipBLASLt has no
@@ -260,6 +363,7 @@ int run_gemm(void *handle, int type, int transA, int transB, int M, int N, int K
     if (bias) {
         LT_TRY(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof bias));
     }
+    if (!p.tuned) tune_plan(ctx, key, p, alpha, A, B, C);
     LT_TRY(hipblasLtMatmul(ctx->lt, p.desc, &alpha, A, p.a, B, p.b, &beta, C, p.c, C, p.c, &p.algo, ctx->workspace,
                            kWorkspaceBytes, ctx->stream));
     return 0;
@@ -381,6 +485,8 @@ int cubert_blas_destroy(void *handle) {
     (void) hipFree(ctx->workspace);
     (void) hipFree(ctx->skinny_partials);
     (void) hipFree(ctx->skinny_counters);
+    if (ctx->tune_start) (void) hipEventDestroy(ctx->tune_start);
+    if (ctx->tune_stop) (void) hipEventDestroy(ctx->tune_stop);
     hipblasLtDestroy(ctx->lt);
     delete ctx;
     return 0;
