@@ -77,6 +77,9 @@ SIGNATURES = {
     "cubert_stream_create": (vp, []),
     "cubert_stream_destroy": (ci, [vp]),
     "cubert_stream_synchronize": (ci, [vp]),
+    "cubert_malloc_host": (vp, [ctypes.c_size_t]),
+    "cubert_free_host": (ci, [vp]),
+    "cubert_event_synchronize": (ci, [vp]),
     "cubert_event_create": (vp, []),
     "cubert_event_destroy": (ci, [vp]),
     "cubert_event_record": (ci, [vp, vp]),

@@ -1,10 +1,17 @@
 #include "Bert.h"
 
+#include <cstring>
 #include <iostream>
 #include <stdexcept>
 #include <vector>
 
 namespace cuBERT {
+
+namespace {
+inline size_t round_up_16(size_t n) { return (n + 15) & ~size_t(15); }
+// bytes of the input block for M tokens: int ids, then int8 mask, then int8 segment ids, each 16-byte aligned
+inline size_t input_block_bytes(size_t M) { return round_up_16(round_up_16(sizeof(int) * M) + M) + M; }
+}  // namespace
 
 template <typename T>
 Bert<T>::Bert(const std::unordered_map<std::string, T *> &var, size_t max_batch_size, size_t seq_length,
@@ -48,11 +55,18 @@ Bert<T>::Bert(const std::unordered_map<std::string, T *> &var, size_t max_batch_
     layout_buffers();
     buffers.allocate();
     layout_buffers();
+
+    input_staging = static_cast<unsigned char *>(cubert_malloc_host(input_block_bytes(max_batch_size * seq_length)));
+    if (input_staging == nullptr) throw std::runtime_error("no page-locked host memory for the request inputs");
+    input_copied = cubert_event_create();
+    if (input_copied == nullptr) throw std::runtime_error("hipEventCreate failed");
 }
 
 template <typename T>
 Bert<T>::~Bert() {
     cuBERT::cuda_stream_synchronize(stream);
+    cubert_event_destroy(input_copied);
+    cubert_free_host(input_staging);
     delete transformer;
     cuBERT::blas_destroy(cublas);
     cuBERT::cuda_stream_destroy(stream);
@@ -75,9 +89,8 @@ void Bert<T>::layout_weights(size_t vocab_size, size_t type_vocab_size) {
 template <typename T>
 void Bert<T>::layout_buffers() {
     const size_t M = max_batch_size * seq_length;
-    input_ids_buf = buffers.take<int>(M);
-    input_mask_buf = buffers.take<int8_t>(M);
-    segment_ids_buf = buffers.take<int8_t>(M);
+    input_block = buffers.take<unsigned char>(input_block_bytes(M));
+    input_ids_buf = nullptr, input_mask_buf = nullptr, segment_ids_buf = nullptr;  // set per request
     _embedding_output = buffers.take<T>(M * hidden_size);
     _pooled_output = buffers.take<T>(max_batch_size * hidden_size);
     _logits = has_classifier ? buffers.take<T>(max_batch_size * num_labels) : nullptr;
@@ -95,9 +108,20 @@ void Bert<T>::compute(size_t batch_size, int *input_ids, int8_t *input_mask, int
         return;
     }
     const size_t M = batch_size * seq_length;
-    cuBERT::memcpyAsync(input_ids_buf, input_ids, sizeof(int) * M, 1, stream);
-    cuBERT::memcpyAsync(input_mask_buf, input_mask, sizeof(int8_t) * M, 1, stream);
-    cuBERT::memcpyAsync(segment_ids_buf, segment_ids, sizeof(int8_t) * M, 1, stream);
+    const size_t mask_at = round_up_16(sizeof(int) * M), segments_at = round_up_16(mask_at + M);
+    if (input_copy_pending) {  // the staging memory may still be being read by the previous request's copy
+        CUBERT_CHECK(cubert_event_synchronize(input_copied));
+        input_copy_pending = false;
+    }
+    std::memcpy(input_staging, input_ids, sizeof(int) * M);
+    std::memcpy(input_staging + mask_at, input_mask, M);
+    std::memcpy(input_staging + segments_at, segment_ids, M);
+    cuBERT::memcpyAsync(input_block, input_staging, segments_at + M, 1, stream);
+    CUBERT_CHECK(cubert_event_record(input_copied, stream));
+    input_copy_pending = true;
+    input_ids_buf = reinterpret_cast<int *>(input_block);
+    input_mask_buf = reinterpret_cast<int8_t *>(input_block + mask_at);
+    segment_ids_buf = reinterpret_cast<int8_t *>(input_block + segments_at);
     forward(batch_size);
 }
 
@@ -108,6 +132,7 @@ void Bert<T>::compute_resident(size_t batch_size) {
     } else if (batch_size == 0) {
         return;
     }
+    if (input_ids_buf == nullptr) throw std::invalid_argument("compute_resident needs a compute call before it");
     forward(batch_size);
 }
 

@@ -82,6 +82,13 @@ private:
     T *output_weights, *output_bias;
 
     Arena buffers;
+    // The three inputs of a request travel as one block: ids, then the mask, then the segment ids, each
+    // starting at a multiple of 16 bytes.  A request is packed into page-locked host memory in that layout and
+    // reaches the device in a single asynchronous copy; the pointers below are set per request.
+    unsigned char *input_block;          // device
+    unsigned char *input_staging = nullptr;  // page-locked host memory, same size
+    void *input_copied = nullptr;        // event: the last copy out of input_staging has finished
+    bool input_copy_pending = false;
     int *input_ids_buf;
     int8_t *input_mask_buf;
     int8_t *segment_ids_buf;

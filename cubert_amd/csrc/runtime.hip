@@ -437,6 +437,19 @@ void *cubert_event_create(void) {
     return e;
 }
 
+void *cubert_malloc_host(size_t size) {
+    void *p = nullptr;
+    if (hipHostMalloc(&p, size, hipHostMallocDefault) != hipSuccess) {
+        (void) hipGetLastError();
+        return nullptr;
+    }
+    return p;
+}
+
+int cubert_free_host(void *ptr) { return ptr ? hip_rc(hipHostFree(ptr)) : 0; }
+
+int cubert_event_synchronize(void *event) { return hip_rc(hipEventSynchronize((hipEvent_t) event)); }
+
 int cubert_event_destroy(void *event) { return event ? hip_rc(hipEventDestroy((hipEvent_t) event)) : 0; }
 
 int cubert_event_record(void *event, void *stream) { return hip_rc(hipEventRecord((hipEvent_t) event, (hipStream_t) stream)); }

@@ -161,9 +161,15 @@ void *cubert_stream_create(void);
 int cubert_stream_destroy(void *stream);
 int cubert_stream_synchronize(void *stream);
 
-/* Timing events on a stream (no counterpart in the reference, which has no built-in profiling):
- * used to measure single kernels of a forward pass where they run. */
+/* Page-locked host memory, for staging buffers that asynchronous copies read or write directly
+ * (the reference copies from the caller's pageable memory, src/cuBERT/common.cpp:176-195). */
+void *cubert_malloc_host(size_t size); /* NULL on failure */
+int cubert_free_host(void *ptr);
+
+/* Events on a stream (no counterpart in the reference, which has no built-in profiling): they time single
+ * kernels of a forward pass where they run and tell the host when a staging buffer may be written again. */
 void *cubert_event_create(void);
+int cubert_event_synchronize(void *event); /* blocks the calling thread until the event has completed */
 int cubert_event_destroy(void *event);
 int cubert_event_record(void *event, void *stream);
 int cubert_event_elapsed_ms(void *start, void *stop, float *ms); /* both events must have completed */
