@@ -150,7 +150,10 @@ class Blas(object):
             self.handle = None
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except Exception:  # interpreter shutdown: module globals may already be gone
+            pass
 
     def gemm(self, transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, bias=None):
         """Column-major C = alpha op(A) op(B) + beta C (+ bias per row of C) on flat tensors."""
