@@ -52,7 +52,8 @@ public:
 
 private:
     struct Layer {
-        T *qkv_kernel, *qkv_bias;            // [hidden, 3*hidden], [3*hidden]
+        // Dense kernels are [in, out] as in the model file, or [out, in] when transposed_kernels is set
+        T *qkv_kernel, *qkv_bias;            // [hidden, 3*hidden] (query | key | value side by side), [3*hidden]
         T *attention_output_kernel, *attention_output_bias;
         T *attention_norm_beta, *attention_norm_gamma;
         T *intermediate_kernel, *intermediate_bias;
@@ -75,6 +76,7 @@ private:
     Profiler *profiler = nullptr;
     bool dense_gelu_fits = true;       // cleared when the few-token Dense + GELU kernel declines this model's shape
     bool keep_packed = false;          // Dense kernels are also kept in the few-token kernel's order
+    bool transposed_kernels = false;   // Dense kernels are stored [out, in] instead of [in, out] (half precision)
     bool fused_attention_fits = true;  // cleared when the one-launch attention kernel declines this model's shape
     size_t max_batch_size, seq_length, hidden_size, num_hidden_layers, num_attention_heads, intermediate_size;
 

@@ -109,6 +109,13 @@ inline void pack_few_token_weights(void *handle, const half *A, int lda, int M, 
     CUBERT_CHECK(cubert_gemm_skinny_pack_f16(handle, h(A), lda, M, K, h(packed)));
 }
 
+inline void transpose(const float *in, int rows, int cols, float *out, void *stream) {
+    CUBERT_CHECK(cubert_transpose_f32(in, rows, cols, out, stream));
+}
+inline void transpose(const half *in, int rows, int cols, half *out, void *stream) {
+    CUBERT_CHECK(cubert_transpose_f16(h(in), rows, cols, h(out), stream));
+}
+
 inline void blas_gemm_strided_batch(void *handle, bool TransA, bool TransB, int m, int n, int k, float alpha,
                                     const float *A, int lda, long long strideA, const float *B, int ldb,
                                     long long strideB, float beta, float *C, int ldc, long long strideC,

@@ -186,6 +186,34 @@ int gather(const Id *ids, int n, const T *table, int width, T *out, void *stream
     return launch(gather_kernel<T, Id, 1>, grid, block, s, ids, n, table, width, out);
 }
 
+// out[c, r] = in[r, c] for a row-major [rows, cols] matrix: 32 x 32 tiles through LDS so that both the reads
+// and the writes are contiguous runs.  Run once per weight matrix when a model is loaded.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void transpose_kernel(const T *__restrict__ in, int rows, int cols,
+                                                           T *__restrict__ out) {
+    __shared__ T tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8 threads
+    const int r0 = blockIdx.y * 32, c0 = blockIdx.x * 32;
+#pragma unroll
+    for (int j = ty; j < 32; j += 8) {
+        if (r0 + j < rows && c0 + tx < cols) tile[j][tx] = in[(size_t) (r0 + j) * cols + c0 + tx];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = ty; j < 32; j += 8) {
+        if (c0 + j < cols && r0 + tx < rows) out[(size_t) (c0 + j) * rows + r0 + tx] = tile[tx][j];
+    }
+}
+
+template <typename T>
+int transpose(const T *in, int rows, int cols, T *out, void *stream) {
+    if (rows < 0 || cols < 0 || !in || !out || in == out) return CUBERT_BAD_ARGUMENT;
+    if (rows == 0 || cols == 0) return 0;
+    dim3 grid((cols + 31) / 32, (rows + 31) / 32);
+    if (grid.y > 65535) return CUBERT_UNSUPPORTED;
+    return launch(transpose_kernel<T>, grid, dim3(kBlock), (hipStream_t) stream, in, rows, cols, out);
+}
+
 }  // namespace
 }  // namespace cubert
 
@@ -224,4 +252,10 @@ extern "C" int cubert_gather_i8_f32(const int8_t *ids, int n, const float *table
 extern "C" int cubert_gather_i8_f16(const int8_t *ids, int n, const cubert_half *table, int width, cubert_half *out,
                                     void *stream) {
     return cubert::gather<half_t, int8_t>(ids, n, (const half_t *) table, width, (half_t *) out, stream);
+}
+extern "C" int cubert_transpose_f32(const float *in, int rows, int cols, float *out, void *stream) {
+    return cubert::transpose<float>(in, rows, cols, out, stream);
+}
+extern "C" int cubert_transpose_f16(const cubert_half *in, int rows, int cols, cubert_half *out, void *stream) {
+    return cubert::transpose<half_t>((const half_t *) in, rows, cols, (half_t *) out, stream);
 }

@@ -30,6 +30,16 @@ __device__ __forceinline__ void ln_stats(float sum, float sumsq, int hidden, flo
     rstd = 1.f / sqrtf(var + 1e-12f);
 }
 
+// One int8 at a wavefront-uniform index, read as the aligned 32-bit word that holds it: a scalar load like the
+// one for a row's id, where a byte load would be a vector load whose latency the dependent row address waits for.
+// (The word is the element's own aligned 4 bytes, so it cannot reach into an unmapped page.)
+__device__ __forceinline__ int uniform_i8(const int8_t *__restrict__ p, int index) {
+    const int8_t *at = p + index;
+    const int within = (int) (reinterpret_cast<uintptr_t>(at) & 3);
+    const uint32_t word = *reinterpret_cast<const uint32_t *>(at - within);
+    return (int) (int8_t) (word >> (within * 8));
+}
+
 // ---- fast path: hidden == 64 * VEC * CHUNKS, everything 16-byte friendly ----
 
 // Normalise the row held in x[][] and store it.  gamma/beta were loaded before
@@ -105,25 +115,30 @@ __global__ __launch_bounds__(kBlock) void embed_ln_kernel(const int32_t *__restr
     const int row = blockIdx.x * kRowsPerBlock + wave_in_block();
     if (row >= rows) return;
     const int lane = threadIdx.x & (kWave - 1);
-    // row is wavefront-uniform, so these are scalar loads
-    const T *w = word + (size_t) ids[row] * H;
-    const T *t = type + (size_t) segments[row] * H;
+    // row is wavefront-uniform, so the id and the segment id arrive through scalar loads; the loads that do not
+    // depend on them (position row, gamma, beta) are issued while those two are on their way
+    const int id = ids[row];
+    const int segment = uniform_i8(segments, row);
     const T *p = pos + (size_t) (row % seq_length) * H;
 
     Vec<T, VEC> a[CHUNKS], b[CHUNKS], d[CHUNKS], g[CHUNKS], be[CHUNKS];
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         const int col = (c * kWave + lane) * VEC;
-        a[c] = load_vec<T, VEC>(w + col);
         b[c] = load_vec<T, VEC>(p + col);
-        d[c] = load_vec<T, VEC>(t + col);
-    }
-#pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
-        const int col = (c * kWave + lane) * VEC;
         g[c] = load_vec<T, VEC>(gamma + col);
         be[c] = load_vec<T, VEC>(beta + col);
     }
+    asm volatile("" ::: "memory");
+    const T *w = word + (size_t) id * H;
+    const T *t = type + (size_t) segment * H;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int col = (c * kWave + lane) * VEC;
+        a[c] = load_vec<T, VEC>(w + col);
+        d[c] = load_vec<T, VEC>(t + col);
+    }
+    asm volatile("" ::: "memory");  // every load is issued before the first conversion
     float x[CHUNKS][VEC];
     float sum = 0.f, sumsq = 0.f;
 #pragma unroll

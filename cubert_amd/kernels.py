@@ -135,6 +135,14 @@ def mean_pool(x):
     return out
 
 
+def transpose(x):
+    """The transpose of a row-major 2-D tensor, as a new contiguous tensor."""
+    rows, cols = x.shape
+    out = torch.empty((cols, rows), dtype=x.dtype, device=x.device)
+    _call("cubert_transpose", x, _ptr(x), rows, cols, _ptr(out), _stream())
+    return out
+
+
 class Blas(object):
     """A BLAS context of the runtime bound to torch's current stream."""
 

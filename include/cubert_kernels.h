@@ -144,6 +144,12 @@ int cubert_mean_pool_f32(const float *in, float *out, int batch, int seq_length,
 int cubert_mean_pool_f16(const cubert_half *in, cubert_half *out, int batch, int seq_length, int hidden,
                          void *stream);
 
+/* out[c, r] = in[r, c] for a row-major [rows, cols] matrix (out must not alias in).  No counterpart in the
+ * reference, which keeps every Dense kernel [in, out] (op/Dense.cpp:47-57): half-precision models here store
+ * them [out, in], the operand order the library's fp16 GEMMs run fastest on. */
+int cubert_transpose_f32(const float *in, int rows, int cols, float *out, void *stream);
+int cubert_transpose_f16(const cubert_half *in, int rows, int cols, cubert_half *out, void *stream);
+
 /* ------------------------------------------------------------------ runtime
  * replaces: reference src/cuBERT/common.h:17-92 (cudart + cuBLAS side). */
 

@@ -305,6 +305,14 @@ def test_gather(K, name, idt):
     assert np.array_equal(got, oracle.embedding(ids, table))  # a copy: bit exact
 
 
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("rows,cols", [(768, 2304), (3072, 768), (33, 65), (1, 7), (100, 1), (32, 32)])
+def test_transpose(K, name, rows, cols):
+    x = q(np.random.default_rng(rows + cols).normal(0, 1, (rows, cols)), name)
+    got = host(K.transpose(dev(x, tdt(name))))
+    assert got.shape == (cols, rows) and np.array_equal(got, x.T)  # a copy: bit exact
+
+
 # ------------------------------------------------------------------ attention contractions (matrix-core kernels)
 
 @pytest.mark.parametrize("name", ["f32", "f16"])
