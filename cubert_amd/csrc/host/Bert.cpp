@@ -19,57 +19,68 @@ Bert<T>::Bert(const std::unordered_map<std::string, T *> &var, size_t max_batch_
               size_t num_attention_heads, size_t intermediate_size, size_t num_labels)
         : max_batch_size(max_batch_size), seq_length(seq_length), hidden_size(hidden_size), num_labels(num_labels),
           transformer(nullptr), _sequence_output(nullptr) {
-    this->stream = cuBERT::cuda_stream_create();
-    this->cublas = cuBERT::blas_create();
-    cuBERT::blas_set_stream(cublas, stream);
+    try {
+        this->stream = cuBERT::cuda_stream_create();
+        this->cublas = cuBERT::blas_create();
+        cuBERT::blas_set_stream(cublas, stream);
 
-    has_pooler_dense = var.count("bert/pooler/dense/kernel") != 0;
-    has_classifier = var.count("output_weights") != 0;
-    has_classifier_bias = has_classifier && var.count("output_bias") != 0;
+        has_pooler_dense = var.count("bert/pooler/dense/kernel") != 0;
+        has_classifier = var.count("output_weights") != 0;
+        has_classifier_bias = has_classifier && var.count("output_bias") != 0;
 
-    const size_t H = hidden_size;
-    layout_weights(vocab_size, type_vocab_size);
-    weights.allocate();
-    layout_weights(vocab_size, type_vocab_size);
+        const size_t H = hidden_size;
+        layout_weights(vocab_size, type_vocab_size);
+        weights.allocate();
+        layout_weights(vocab_size, type_vocab_size);
 
-    cuBERT::memcpy(word_embeddings, var.at("bert/embeddings/word_embeddings"), vocab_size * H * sizeof(T), 1);
-    cuBERT::memcpy(token_type_embeddings, var.at("bert/embeddings/token_type_embeddings"),
-                   type_vocab_size * H * sizeof(T), 1);
-    // only the positions a sequence of seq_length tokens can use are kept on the device
-    cuBERT::memcpy(position_embeddings, var.at("bert/embeddings/position_embeddings"), seq_length * H * sizeof(T), 1);
-    cuBERT::memcpy(embedding_norm_beta, var.at("bert/embeddings/LayerNorm/beta"), H * sizeof(T), 1);
-    cuBERT::memcpy(embedding_norm_gamma, var.at("bert/embeddings/LayerNorm/gamma"), H * sizeof(T), 1);
-    if (has_pooler_dense) {
-        cuBERT::memcpy(pooler_kernel, var.at("bert/pooler/dense/kernel"), H * H * sizeof(T), 1);
-        cuBERT::memcpy(pooler_bias, var.at("bert/pooler/dense/bias"), H * sizeof(T), 1);
+        cuBERT::memcpy(word_embeddings, var.at("bert/embeddings/word_embeddings"), vocab_size * H * sizeof(T), 1);
+        cuBERT::memcpy(token_type_embeddings, var.at("bert/embeddings/token_type_embeddings"),
+                       type_vocab_size * H * sizeof(T), 1);
+        // only the positions a sequence of seq_length tokens can use are kept on the device
+        cuBERT::memcpy(position_embeddings, var.at("bert/embeddings/position_embeddings"), seq_length * H * sizeof(T), 1);
+        cuBERT::memcpy(embedding_norm_beta, var.at("bert/embeddings/LayerNorm/beta"), H * sizeof(T), 1);
+        cuBERT::memcpy(embedding_norm_gamma, var.at("bert/embeddings/LayerNorm/gamma"), H * sizeof(T), 1);
+        if (has_pooler_dense) {
+            cuBERT::memcpy(pooler_kernel, var.at("bert/pooler/dense/kernel"), H * H * sizeof(T), 1);
+            cuBERT::memcpy(pooler_bias, var.at("bert/pooler/dense/bias"), H * sizeof(T), 1);
+        }
+        if (has_classifier) {
+            cuBERT::memcpy(output_weights, var.at("output_weights"), num_labels * H * sizeof(T), 1);
+            if (has_classifier_bias) cuBERT::memcpy(output_bias, var.at("output_bias"), num_labels * sizeof(T), 1);
+        }
+
+        this->transformer = new Transformer<T>(cublas, "bert/encoder", var, max_batch_size, seq_length, hidden_size,
+                                               num_hidden_layers, num_attention_heads, intermediate_size);
+        this->transformer->set_profiler(&profiler);
+
+        layout_buffers();
+        buffers.allocate();
+        layout_buffers();
+
+        input_staging = static_cast<unsigned char *>(cubert_malloc_host(input_block_bytes(max_batch_size * seq_length)));
+        if (input_staging == nullptr) throw std::runtime_error("no page-locked host memory for the request inputs");
+        input_copied = cubert_event_create();
+        if (input_copied == nullptr) throw std::runtime_error("hipEventCreate failed");
+    } catch (...) {
+        release();
+        throw;
     }
-    if (has_classifier) {
-        cuBERT::memcpy(output_weights, var.at("output_weights"), num_labels * H * sizeof(T), 1);
-        if (has_classifier_bias) cuBERT::memcpy(output_bias, var.at("output_bias"), num_labels * sizeof(T), 1);
-    }
-
-    this->transformer = new Transformer<T>(cublas, "bert/encoder", var, max_batch_size, seq_length, hidden_size,
-                                           num_hidden_layers, num_attention_heads, intermediate_size);
-    this->transformer->set_profiler(&profiler);
-
-    layout_buffers();
-    buffers.allocate();
-    layout_buffers();
-
-    input_staging = static_cast<unsigned char *>(cubert_malloc_host(input_block_bytes(max_batch_size * seq_length)));
-    if (input_staging == nullptr) throw std::runtime_error("no page-locked host memory for the request inputs");
-    input_copied = cubert_event_create();
-    if (input_copied == nullptr) throw std::runtime_error("hipEventCreate failed");
 }
 
 template <typename T>
 Bert<T>::~Bert() {
-    cuBERT::cuda_stream_synchronize(stream);
-    cubert_event_destroy(input_copied);
+    release();
+}
+
+template <typename T>
+void Bert<T>::release() noexcept {
+    if (stream != nullptr) cubert_stream_synchronize(stream);
+    cubert_event_destroy(input_copied);  // null is accepted by these three
     cubert_free_host(input_staging);
     delete transformer;
-    cuBERT::blas_destroy(cublas);
-    cuBERT::cuda_stream_destroy(stream);
+    if (cublas != nullptr) cubert_blas_destroy(cublas);
+    if (stream != nullptr) cubert_stream_destroy(stream);
+    input_copied = nullptr, input_staging = nullptr, transformer = nullptr, cublas = nullptr, stream = nullptr;
 }
 
 template <typename T>

@@ -63,16 +63,17 @@ public:
 
 private:
     void forward(size_t batch_size);
+    void release() noexcept;  // everything the constructor acquired so far (also run when it throws)
     void layout_weights(size_t vocab_size, size_t type_vocab_size);
     void layout_buffers();
 
-    void *cublas;
-    void *stream;
+    void *cublas = nullptr;
+    void *stream = nullptr;
 
     size_t max_batch_size, seq_length, hidden_size, num_labels;
     bool has_pooler_dense, has_classifier, has_classifier_bias;
 
-    Transformer<T> *transformer;
+    Transformer<T> *transformer = nullptr;
     Profiler profiler;
 
     Arena weights;

@@ -69,10 +69,10 @@ BertM<T>::BertM(const char *model_file, size_t max_batch_size, size_t seq_length
         const auto start = std::chrono::high_resolution_clock::now();
         cuBERT::set_gpu(device);
         cuBERT::gpu_info(device);
-        bert_instances.push_back(new Bert<T>(graph.var, max_batch_size, seq_length, graph.vocab_size,
-                                             graph.type_vocab_size, graph.hidden_size, num_hidden_layers,
-                                             num_attention_heads, graph.intermediate_size, graph.num_labels));
-        mutex_instances.push_back(new std::mutex());
+        bert_instances.emplace_back(new Bert<T>(graph.var, max_batch_size, seq_length, graph.vocab_size,
+                                                graph.type_vocab_size, graph.hidden_size, num_hidden_layers,
+                                                num_attention_heads, graph.intermediate_size, graph.num_labels));
+        mutex_instances.emplace_back(new std::mutex());
         const auto finish = std::chrono::high_resolution_clock::now();
         std::cerr << "device setup: " << device << ". Took "
                   << std::chrono::duration_cast<std::chrono::milliseconds>(finish - start).count() << " milliseconds."
@@ -84,9 +84,8 @@ template <typename T>
 BertM<T>::~BertM() {
     for (size_t i = 0; i < bert_instances.size(); ++i) {
         cuBERT::set_gpu((int) i);
-        delete bert_instances[i];
+        bert_instances[i].reset();
     }
-    for (auto *m : mutex_instances) delete m;
 }
 
 template <typename T>
@@ -96,7 +95,7 @@ unsigned int BertM<T>::compute(size_t batch_size, int *input_ids, int8_t *input_
     const unsigned int choice = count % bert_instances.size();
 
     cuBERT::set_gpu((int) choice);
-    Bert<T> *bert = bert_instances[choice];
+    Bert<T> *bert = bert_instances[choice].get();
     std::lock_guard<std::mutex> lg(*mutex_instances[choice]);
 
     bert->compute(batch_size, input_ids, input_mask, segment_ids);
@@ -118,7 +117,7 @@ unsigned int BertM<T>::compute(size_t batch_size, int *input_ids, int8_t *input_
     const unsigned int choice = count % bert_instances.size();
 
     cuBERT::set_gpu((int) choice);
-    Bert<T> *bert = bert_instances[choice];
+    Bert<T> *bert = bert_instances[choice].get();
     std::lock_guard<std::mutex> lg(*mutex_instances[choice]);
 
     bert->compute(batch_size, input_ids, input_mask, segment_ids);

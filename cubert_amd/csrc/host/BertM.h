@@ -7,6 +7,7 @@
 
 #include <atomic>
 #include <cstdint>
+#include <memory>
 #include <mutex>
 #include <vector>
 
@@ -36,12 +37,13 @@ public:
     // Shape facts read from the model file, for callers that size output buffers.
     size_t hidden_size() const { return graph.hidden_size; }
     size_t num_labels() const { return graph.num_labels; }
-    Bert<T> *replica(size_t i) { return bert_instances[i]; }
+    Bert<T> *replica(size_t i) { return bert_instances[i].get(); }
 
 private:
     Graph<T> graph;
-    std::vector<Bert<T> *> bert_instances;
-    std::vector<std::mutex *> mutex_instances;
+    // owned: a constructor that throws half way (a later device fails) releases the replicas built so far
+    std::vector<std::unique_ptr<Bert<T>>> bert_instances;
+    std::vector<std::unique_ptr<std::mutex>> mutex_instances;
     std::atomic<uint8_t> rr;
 };
 

@@ -12,6 +12,17 @@ template <typename T>
 void upload(T *dst, const T *src, size_t count) {
     if (dst != nullptr) cuBERT::memcpy(dst, src, count * sizeof(T), 1);
 }
+
+// device memory for the duration of a scope (a missing weight name throws out of the constructor)
+struct ScopedDeviceBuffer {
+    void *ptr = nullptr;
+    explicit ScopedDeviceBuffer(size_t bytes) : ptr(bytes ? cuBERT::malloc(bytes) : nullptr) {}
+    ScopedDeviceBuffer(const ScopedDeviceBuffer &) = delete;
+    ScopedDeviceBuffer &operator=(const ScopedDeviceBuffer &) = delete;
+    ~ScopedDeviceBuffer() {
+        if (ptr != nullptr) cubert_free(ptr);
+    }
+};
 }  // namespace
 
 template <typename T>
@@ -42,7 +53,8 @@ Transformer<T>::Transformer(void *cublas, const std::string &var_prefix,
 
     void *stream = cuBERT::blas_get_stream(cublas);
     const size_t largest = H * (3 * H > I ? 3 * H : I);
-    T *staging = transposed_kernels ? static_cast<T *>(cuBERT::malloc(largest * sizeof(T))) : nullptr;
+    ScopedDeviceBuffer staging_memory(transposed_kernels ? largest * sizeof(T) : 0);
+    T *staging = static_cast<T *>(staging_memory.ptr);
     // one Dense kernel, [in, out] on the host, into its place on the device (and its few-token copy)
     auto load_kernel = [&](T *dst, T *few_token_copy, const T *host, size_t in, size_t out) {
         T *plain = transposed_kernels ? staging : dst;
@@ -84,10 +96,7 @@ Transformer<T>::Transformer(void *cublas, const std::string &var_prefix,
         upload(w.output_norm_beta, var.at(p + "/output/LayerNorm/beta"), H);
         upload(w.output_norm_gamma, var.at(p + "/output/LayerNorm/gamma"), H);
     }
-    if (staging != nullptr) {
-        cuBERT::cuda_stream_synchronize(stream);
-        cuBERT::free(staging);
-    }
+    cuBERT::cuda_stream_synchronize(stream);  // nothing reads the staging buffer after this
 
     layout_buffers();
     buffers.allocate();
