@@ -48,7 +48,7 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_pack_kernel(const T *__res
     packed[idx] = feature < M ? A[(size_t) k * lda + feature] : from_f32<T>(0.f);
 }
 
-template <typename T, bool GELU, bool PACKED>
+template <typename T, bool GELU, bool PACKED, int PASSES>
 __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__restrict__ A, int lda,
                                                                      const T *__restrict__ B, int ldb,
                                                                      const T *__restrict__ bias, T *__restrict__ C,
@@ -66,32 +66,44 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
     const int c_end = c_begin + chunks_per_slice < chunks ? c_begin + chunks_per_slice : chunks;
 
     v16f32 acc = v16f32{};
-    for (int c = c_begin + wave; c < c_end; c += kSkinnyWaves) {
+    for (int c0 = c_begin + wave; c0 < c_end; c0 += kSkinnyWaves * PASSES) {
         // reduction slot of MFMA t in lane half hh is k = c*16 + hh*8 + t: the token operand of a lane is 8
-        // consecutive values of one row of B (vector loads), the weight operand one column of 8 rows of A
-        const int kb = c * kSkinnyChunk + hh * 8;
-        float x[8], w[8];
+        // consecutive values of one row of B (vector loads), the weight operand one column of 8 rows of A.
+        // The loads of all PASSES chunks are issued before the first MFMA; a chunk past the slice is read
+        // from the wavefront's first chunk (a valid address, no branch around the loads) with its tokens zeroed.
+        float x[PASSES][8], w[PASSES][8];
 #pragma unroll
-        for (int u = 0; u < 8 / V; ++u) {
-            Vec<T, V> xv = Vec<T, V>{};
-            if (r < N) xv = load_vec<T, V>(B + (size_t) r * ldb + kb + u * V);
-#pragma unroll
-            for (int e = 0; e < V; ++e) x[u * V + e] = to_f32(xv.v[e]);
-        }
-        if (PACKED) {
-            const T *src = A + (((size_t) blockIdx.x * chunks + c) * kWave + lane) * 8;
+        for (int p = 0; p < PASSES; ++p) {
+            const int c = c0 + p * kSkinnyWaves;
+            const bool inside = c < c_end;
+            const int kb = (inside ? c : c0) * kSkinnyChunk + hh * 8;
 #pragma unroll
             for (int u = 0; u < 8 / V; ++u) {
-                const Vec<T, V> wv = load_vec<T, V>(src + u * V);
+                Vec<T, V> xv = Vec<T, V>{};
+                if (r < N) xv = load_vec<T, V>(B + (size_t) r * ldb + kb + u * V);
 #pragma unroll
-                for (int e = 0; e < V; ++e) w[u * V + e] = to_f32(wv.v[e]);
+                for (int e = 0; e < V; ++e) x[p][u * V + e] = inside ? to_f32(xv.v[e]) : 0.f;
             }
-        } else {
+            if (PACKED) {
+                const T *src = A + (((size_t) blockIdx.x * chunks + (inside ? c : c0)) * kWave + lane) * 8;
 #pragma unroll
-            for (int t = 0; t < 8; ++t) w[t] = feature < M ? to_f32(A[(size_t) (kb + t) * lda + feature]) : 0.f;
+                for (int u = 0; u < 8 / V; ++u) {
+                    const Vec<T, V> wv = load_vec<T, V>(src + u * V);
+#pragma unroll
+                    for (int e = 0; e < V; ++e) w[p][u * V + e] = to_f32(wv.v[e]);
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    w[p][t] = feature < M ? to_f32(A[(size_t) (kb + t) * lda + feature]) : 0.f;
+                }
+            }
         }
 #pragma unroll
-        for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[t], w[t], acc, 0, 0, 0);
+        for (int p = 0; p < PASSES; ++p) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[p][t], w[p][t], acc, 0, 0, 0);
+        }
     }
     // lane holds C[feature = m0 + r, token = acc_row(i, hh)]
 #pragma unroll
@@ -162,18 +174,33 @@ int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, int packe
     if (!is_aligned(B, 16) || (ldb * sizeof(T)) % 16 != 0) return CUBERT_UNSUPPORTED;
     const int blocks = (M + 31) / 32;
     const int chunks = K / kSkinnyChunk;
-    // one pass per wavefront unless that would need more slices than the workspace holds
+    // One pass (16 reduction values) per wavefront, unless that makes more workgroups than the chip has compute
+    // units: a second round of workgroups costs more than a second pass of every wavefront (measured at
+    // 768 x 3072 and 3072 x 768: 10.3 -> 9.5 us), while fewer, longer workgroups lose where one round is enough
+    // (768 x 768: 6.4 -> 8.1 us).  Not for 2-byte weights in the plain layout, whose 2-byte loads make the
+    // second pass expensive (10.1 -> 11.5 us).  More passes still when the workspace cannot hold that many slices.
+    constexpr int kComputeUnits = 256;
     int chunks_per_slice = kSkinnyWaves;
     int slices = (chunks + chunks_per_slice - 1) / chunks_per_slice;
+    if (slices > 1 && (long long) slices * blocks > kComputeUnits && (packed || sizeof(T) == 4)) {
+        chunks_per_slice = 2 * kSkinnyWaves;
+        slices = (chunks + chunks_per_slice - 1) / chunks_per_slice;
+    }
     while (slices > 1 && (size_t) slices * 32 * blocks * 32 > partial_floats) {
         chunks_per_slice += kSkinnyWaves;
         slices = (chunks + chunks_per_slice - 1) / chunks_per_slice;
     }
     if (blocks > 65535 || slices > 65535 || (slices > 1 && blocks > n_counters)) return CUBERT_UNSUPPORTED;
     const dim3 grid(blocks, slices), block(kSkinnyThreads);
-#define CUBERT_SKINNY_LAUNCH(GELU, PACKED)                                                                         \
-    return launch(gemm_skinny_kernel<T, GELU, PACKED>, grid, block, stream, A, lda, B, ldb, bias, C, ldc, M, N, K, \
-                  alpha, partials, counters, chunks_per_slice)
+#define CUBERT_SKINNY_LAUNCH(GELU, PACKED)                                                                           \
+    do {                                                                                                             \
+        if (chunks_per_slice == kSkinnyWaves) {                                                                      \
+            return launch(gemm_skinny_kernel<T, GELU, PACKED, 1>, grid, block, stream, A, lda, B, ldb, bias, C, ldc, M, \
+                          N, K, alpha, partials, counters, chunks_per_slice);                                        \
+        }                                                                                                            \
+        return launch(gemm_skinny_kernel<T, GELU, PACKED, 2>, grid, block, stream, A, lda, B, ldb, bias, C, ldc, M, N, \
+                      K, alpha, partials, counters, chunks_per_slice);                                               \
+    } while (0)
     if (activation == 1) {
         if (packed) CUBERT_SKINNY_LAUNCH(true, true);
         CUBERT_SKINNY_LAUNCH(true, false);

@@ -184,6 +184,25 @@ def test_benchmark_configurations(cb, name, rows):
     np.testing.assert_allclose(seq.var(-1), 1.0, atol=1e-2 if half else 1e-4)
 
 
+def test_sequences_of_a_batch_are_independent_at_full_size(cb):
+    """A size-independent property at a benchmark shape (C2: fp16, batch 32 x seq 128, heavy padding): permuting the
+    sequences of a batch permutes the outputs, and a sequence computed alone gives what it gives inside the batch."""
+    from cubert_amd.testing import CONFIGS, config_inputs, config_weights
+    cfg = CONFIGS["C2"]
+    m = cfg["model"]
+    w = config_weights("C2", seed=0)
+    ids, mask, seg = config_inputs("C2", seed=0)
+    perm = np.random.default_rng(5).permutation(cfg["batch"])
+    bert = cb.Bert(w, cfg["batch"], cfg["seq_length"], m["layers"], m["heads"], 1)
+    first = bert.forward(ids, mask, seg)
+    moved = bert.forward(ids[perm], mask[perm], seg[perm])
+    alone = bert.forward(ids[3:4], mask[3:4], seg[3:4])
+    bert.close()
+    for k in ("pooled_output", "sequence_output"):
+        assert_close(moved[k], first[k][perm], 2e-3, "permuted batch, " + k)
+        assert_close(alone[k], first[k][3:4], 2e-3, "single sequence, " + k)
+
+
 # ------------------------------------------------------------------ the public C API on a GraphDef file
 
 @pytest.fixture(scope="module")
