@@ -465,14 +465,18 @@ def test_gemm_skinny_against_oracle_sgemm(K, name, M, N, K_):
     pre = (oracle.sgemm(0, 0, M, N, K_, 1.0, A, M, B, ldb, 0.0, np.zeros(N * M, np.float32), M).reshape(N, M)
            + bias[None, :])
     assert_close(host(C), oracle.gelu(pre).ravel(), 2e-5 if name == "f32" else 2e-3, "gemm_skinny + gelu %s" % name)
-    # the same on weights packed into the kernel's own order: bit-identical to the unpacked call
+    # the same on weights packed into the kernel's own order: bit-identical to the unpacked call where both cut the
+    # reduction the same way (2-byte weights in the plain layout keep one pass per wavefront at every size)
     packed = blas.gemm_skinny_pack(dA, M, M, K_)
     for gelu in (False, True):
         C1 = torch.zeros((N * M,), dtype=tdt(name), device="cuda")
         C2 = torch.full((N * M,), 3.0, dtype=tdt(name), device="cuda")
         assert blas.gemm_skinny(M, N, K_, 1.0, dA, M, dB, ldb, C1, M, bias=dbias, gelu=gelu) is not None
         assert blas.gemm_skinny_packed(M, N, K_, 1.0, packed, dB, ldb, C2, M, bias=dbias, gelu=gelu) is not None
-        assert torch.equal(C1, C2)
+        if name == "f32":
+            assert torch.equal(C1, C2)
+        else:
+            assert_close(host(C2), host(C1), 2e-3, "packed vs plain weights, gelu=%s" % gelu)
     # the general entry point takes the same path by itself
     C = torch.zeros((N * M,), dtype=tdt(name), device="cuda")
     blas.gemm(0, 0, M, N, K_, 1.0, dA, M, dB, ldb, 0.0, C, M, bias=dbias)
