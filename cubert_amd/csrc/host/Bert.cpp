@@ -59,8 +59,6 @@ Bert<T>::Bert(const std::unordered_map<std::string, T *> &var, size_t max_batch_
 
         input_staging = static_cast<unsigned char *>(cubert_malloc_host(input_block_bytes(max_batch_size * seq_length)));
         if (input_staging == nullptr) throw std::runtime_error("no page-locked host memory for the request inputs");
-        input_copied = cubert_event_create();
-        if (input_copied == nullptr) throw std::runtime_error("hipEventCreate failed");
     } catch (...) {
         release();
         throw;
@@ -75,12 +73,11 @@ Bert<T>::~Bert() {
 template <typename T>
 void Bert<T>::release() noexcept {
     if (stream != nullptr) cubert_stream_synchronize(stream);
-    cubert_event_destroy(input_copied);  // null is accepted by these three
-    cubert_free_host(input_staging);
+    cubert_free_host(input_staging);  // null is accepted
     delete transformer;
     if (cublas != nullptr) cubert_blas_destroy(cublas);
     if (stream != nullptr) cubert_stream_destroy(stream);
-    input_copied = nullptr, input_staging = nullptr, transformer = nullptr, cublas = nullptr, stream = nullptr;
+    input_staging = nullptr, transformer = nullptr, cublas = nullptr, stream = nullptr;
 }
 
 template <typename T>
@@ -112,6 +109,12 @@ template <typename T>
 void Bert<T>::_pre_compute(size_t) {}
 
 template <typename T>
+void Bert<T>::synchronize() {
+    cuBERT::cuda_stream_synchronize(stream);
+    input_copy_pending = false;
+}
+
+template <typename T>
 void Bert<T>::compute(size_t batch_size, int *input_ids, int8_t *input_mask, int8_t *segment_ids) {
     if (batch_size > max_batch_size) {
         throw std::invalid_argument("batch_size > max_batch_size");
@@ -120,15 +123,13 @@ void Bert<T>::compute(size_t batch_size, int *input_ids, int8_t *input_mask, int
     }
     const size_t M = batch_size * seq_length;
     const size_t mask_at = round_up_16(sizeof(int) * M), segments_at = round_up_16(mask_at + M);
-    if (input_copy_pending) {  // the staging memory may still be being read by the previous request's copy
-        CUBERT_CHECK(cubert_event_synchronize(input_copied));
-        input_copy_pending = false;
-    }
+    // The staging memory may still be being read by the previous request's copy when that request's outputs
+    // were never fetched (every output method drains the stream); no event sits on a request's own path.
+    if (input_copy_pending) synchronize();
     std::memcpy(input_staging, input_ids, sizeof(int) * M);
     std::memcpy(input_staging + mask_at, input_mask, M);
     std::memcpy(input_staging + segments_at, segment_ids, M);
     cuBERT::memcpyAsync(input_block, input_staging, segments_at + M, 1, stream);
-    CUBERT_CHECK(cubert_event_record(input_copied, stream));
     input_copy_pending = true;
     input_ids_buf = reinterpret_cast<int *>(input_block);
     input_mask_buf = reinterpret_cast<int8_t *>(input_block + mask_at);
@@ -200,26 +201,26 @@ void Bert<T>::logits(size_t batch_size, T *logits, T *probs) {
     if (has_classifier && probs != nullptr) {
         cuBERT::memcpyAsync(probs, _probs, sizeof(T) * batch_size * num_labels, 2, stream);
     }
-    cuBERT::cuda_stream_synchronize(stream);
+    synchronize();
 }
 
 template <typename T>
 void Bert<T>::pooled_output(size_t batch_size, T *pooled_output) {
     cuBERT::memcpyAsync(pooled_output, _pooled_output, sizeof(T) * batch_size * hidden_size, 2, stream);
-    cuBERT::cuda_stream_synchronize(stream);
+    synchronize();
 }
 
 template <typename T>
 void Bert<T>::sequence_output(size_t batch_size, T *sequence_output) {
     cuBERT::memcpyAsync(sequence_output, _sequence_output, sizeof(T) * batch_size * seq_length * hidden_size, 2, stream);
-    cuBERT::cuda_stream_synchronize(stream);
+    synchronize();
 }
 
 template <typename T>
 void Bert<T>::embedding_output(size_t batch_size, T *embedding_output) {
     cuBERT::memcpyAsync(embedding_output, _embedding_output, sizeof(T) * batch_size * seq_length * hidden_size, 2,
                         stream);
-    cuBERT::cuda_stream_synchronize(stream);
+    synchronize();
 }
 
 template <typename T>
@@ -240,7 +241,7 @@ void Bert<T>::output(size_t batch_size, cuBERT_Output *output) {
     if (output->embedding_output != nullptr) {
         cuBERT::memcpyAsync(output->embedding_output, _embedding_output, sizeof(T) * tokens, 2, stream);
     }
-    cuBERT::cuda_stream_synchronize(stream);
+    synchronize();
 }
 
 template <>

@@ -57,12 +57,13 @@ public:
     // Per-kernel timing: switch kinds on (bit k = Profiler::Kind k), run, synchronise, then read.
     void profile(unsigned kinds) { profiler.enable(kinds); }
     void profile_read(double *total_ms, int *count) {
-        cuBERT::cuda_stream_synchronize(stream);
+        synchronize();
         profiler.collect(total_ms, count);
     }
 
 private:
     void forward(size_t batch_size);
+    void synchronize();       // drains the stream
     void release() noexcept;  // everything the constructor acquired so far (also run when it throws)
     void layout_weights(size_t vocab_size, size_t type_vocab_size);
     void layout_buffers();
@@ -88,8 +89,7 @@ private:
     // reaches the device in a single asynchronous copy; the pointers below are set per request.
     unsigned char *input_block;          // device
     unsigned char *input_staging = nullptr;  // page-locked host memory, same size
-    void *input_copied = nullptr;        // event: the last copy out of input_staging has finished
-    bool input_copy_pending = false;
+    bool input_copy_pending = false;     // a copy out of input_staging was queued and the stream not drained since
     int *input_ids_buf;
     int8_t *input_mask_buf;
     int8_t *segment_ids_buf;
