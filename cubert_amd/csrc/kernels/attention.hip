@@ -451,11 +451,19 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
 // query, so the per-query factors cross lanes through 128 bytes of wavefront-private LDS.  The result is divided
 // by l once at the end (scores and probabilities are not rounded to the storage type one by one as the
 // three-kernel path does; the difference is within the fp16 storage tolerance).
+//
+// Key tiles (32 keys) whose mask is zero throughout are left out altogether -- not loaded, not multiplied: a
+// masked key's score is 10000 below every unmasked one of its query, its exp is exactly 0 in fp32, so it adds
+// nothing to the sum or the context as long as the sequence has one unmasked key (a sequence without any keeps
+// all its tiles: there the shift cancels and the softmax runs over the raw scores, as in the reference).  Every
+// query row, padded or not, is still computed.  skip_masked_tiles = 0 (a mask that cannot be read as 32-bit
+// words) computes all tiles.
 template <typename T, int D>
 __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restrict__ q, const T *__restrict__ k,
                                                                const T *__restrict__ v, int ld,
                                                                const int8_t *__restrict__ mask, T *__restrict__ ctx,
-                                                               int ld_ctx, float alpha, int heads, int seq) {
+                                                               int ld_ctx, float alpha, int heads, int seq,
+                                                               int skip_masked_tiles) {
     constexpr int V = Mma<T>::kVec;
     constexpr int kSteps = D / 2 / V;
     constexpr int kColTiles = D / 32;
@@ -483,14 +491,30 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
 #pragma unroll
     for (int t = 0; t < kSteps; ++t) qv[t] = load_vec<T, V>(q_row + t * V);
 
+    // bit kt: key tile kt has an unmasked key (workgroup-uniform: scalar loads of the mask row as words)
+    unsigned live = 0;
+    if (mask != nullptr && skip_masked_tiles) {
+        const uint32_t *words = reinterpret_cast<const uint32_t *>(mask + (size_t) b * S);
+        for (int kt = 0; kt < KT; ++kt) {
+            uint32_t any = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) any |= words[kt * 8 + i];
+            live |= (any != 0 ? 1u : 0u) << kt;
+        }
+    }
+    if (live == 0) live = KT >= 32 ? ~0u : (1u << KT) - 1u;
+    live = __builtin_amdgcn_readfirstlane(live);
+
     constexpr int kVecPerRow = D / V;
     constexpr int kLoads = D / V / 2;  // vectors per thread for K, slot groups per thread for V^T
     Vec<T, V> kreg[kLoads], vreg[kLoads];
 #pragma unroll
     for (int u = 0; u < kLoads; ++u) {
+        // (the 64 consecutive idx of a wavefront lie in one key tile, so the tests below are wavefront-uniform)
         const int idx = threadIdx.x + u * threads;
         const int row = idx / kVecPerRow, c = idx - row * kVecPerRow;
-        kreg[u] = load_vec<T, V>(k_head + (size_t) row * ld + c * V);
+        kreg[u] = Vec<T, V>{};
+        if ((live >> (row >> 5)) & 1u) kreg[u] = load_vec<T, V>(k_head + (size_t) row * ld + c * V);
     }
 #pragma unroll
     for (int u = 0; u < kLoads; ++u) {
@@ -498,9 +522,12 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
         const int j = idx % D, grp = idx / D;
         const int kt = grp / (32 / V), in_tile = grp % (32 / V);
         const int run = in_tile >> 1, half = in_tile & 1;
+        vreg[u] = Vec<T, V>{};
+        if ((live >> kt) & 1u) {
 #pragma unroll
-        for (int e = 0; e < V; ++e) {
-            vreg[u].v[e] = v_head[(size_t) (kt * 32 + acc_row(run * V + e, half)) * ld + j];
+            for (int e = 0; e < V; ++e) {
+                vreg[u].v[e] = v_head[(size_t) (kt * 32 + acc_row(run * V + e, half)) * ld + j];
+            }
         }
     }
     for (int i = threadIdx.x; i < S; i += threads) {
@@ -529,14 +556,24 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
 #pragma unroll
     for (int jt = 0; jt < kColTiles; ++jt) out[jt] = v16f32{};
 
-    for (int c0 = 0; c0 < KT; c0 += kChunk) {
+    bool first_chunk = true;
+    for (unsigned todo = live; todo != 0;) {  // the live key tiles in ascending order, kChunk per step
+        int tiles[kChunk];
+#pragma unroll
+        for (int cc = 0; cc < kChunk; ++cc) {
+            tiles[cc] = -1;
+            if (todo != 0) {
+                tiles[cc] = __builtin_ctz(todo);
+                todo &= todo - 1;
+            }
+        }
         v16f32 p[kChunk];
         float cm = -3.402823466e+38f;
 #pragma unroll
         for (int cc = 0; cc < kChunk; ++cc) {
-            const int kt = c0 + cc;
+            const int kt = tiles[cc];
             v16f32 c = {};
-            if (kt < KT) {  // wavefront-uniform
+            if (kt >= 0) {  // wavefront-uniform
 #pragma unroll
                 for (int t = 0; t < kSteps; ++t) {
                     Mma<T>::run(c, load_vec<T, V>(s_k + (kt * 32 + r) * kPitchK + hh * (D / 2) + t * V), qv[t]);
@@ -574,7 +611,7 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
         m = m_new;
 
         // rescale the accumulators: row i of a lane is query acc_row(i, hh), whose factor is in lane acc_row(i, hh)
-        if (c0 > 0 && __any(f != 1.f)) {  // wavefront-uniform: skipped when no query's maximum moved
+        if (!first_chunk && __any(f != 1.f)) {  // wavefront-uniform: skipped when no query's maximum moved
             if (hh == 0) factor[r] = f;
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): LDS operations of one wavefront complete in order
             __builtin_amdgcn_wave_barrier();
@@ -589,10 +626,11 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
             }
             __builtin_amdgcn_wave_barrier();  // the reads above come before the next chunk's write
         }
+        first_chunk = false;
 #pragma unroll
         for (int cc = 0; cc < kChunk; ++cc) {
-            const int kt = c0 + cc;
-            if (kt < KT) {
+            const int kt = tiles[cc];
+            if (kt >= 0) {
 #pragma unroll
                 for (int run = 0; run < 16 / V; ++run) {
                     Vec<T, V> a;
@@ -758,8 +796,9 @@ int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask,
     auto kernel = attention_flash_kernel<T, D>;
     static std::atomic<unsigned long long> raised{0};  // per instantiation
     if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
+    const int skip_masked_tiles = mask != nullptr && is_aligned(mask, 4);  // seq is a multiple of 32
     return launch_untimed(kernel, dim3(batch * heads), dim3(seq / 32 * kWave), (unsigned) lds, s, q, k, v, ld, mask,
-                          ctx, ld_ctx, alpha, heads, seq);
+                          ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles);
 }
 
 template <typename T>
