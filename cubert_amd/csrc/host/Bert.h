@@ -8,6 +8,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <string>
+#include <vector>
 #include <unordered_map>
 
 #include "Arena.h"
@@ -64,6 +65,8 @@ public:
 private:
     void forward(size_t batch_size);
     void synchronize();       // drains the stream
+    void fetch(void *dst, const void *src, size_t bytes);  // queue one device-to-host output copy
+    void finish_outputs();    // drain the stream and hand staged outputs to the caller's arrays
     void release() noexcept;  // everything the constructor acquired so far (also run when it throws)
     void layout_weights(size_t vocab_size, size_t type_vocab_size);
     void layout_buffers();
@@ -89,6 +92,15 @@ private:
     // reaches the device in a single asynchronous copy; the pointers below are set per request.
     unsigned char *input_block;          // device
     unsigned char *input_staging = nullptr;  // page-locked host memory, same size
+    // small outputs pass through page-locked memory on their way to the caller's (pageable) arrays
+    static constexpr size_t kOutputStagingBytes = 32 * 1024;
+    struct StagedOutput {
+        void *dst;
+        size_t offset, bytes;
+    };
+    unsigned char *output_staging = nullptr;
+    std::vector<StagedOutput> staged;
+    size_t staged_bytes = 0;
     bool input_copy_pending = false;     // a copy out of input_staging was queued and the stream not drained since
     int *input_ids_buf;
     int8_t *input_mask_buf;
