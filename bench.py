@@ -67,6 +67,8 @@ def algorithmic_bytes(cfg):
         "bias_tanh": 2 * B * H * e + H * e,
         "mean_pool": (M + B) * H * e,
         "row_softmax": 2 * B * cfg["labels"] * e,
+        # pooler bias + tanh, classifier and softmax in one launch: pooled in and out, weights in, logits + probs out
+        "classifier_head": (2 * B * H + H + cfg["labels"] * H + cfg["labels"] + 2 * B * cfg["labels"]) * e,
         # fused attention core (seq_len <= 128): Q, K, V read, context written, the scores never reach memory
         "attention_fused": 4 * M * H * e + B * S,
     }

@@ -106,6 +106,7 @@ for _t in ("f32", "f16"):
         "cubert_bias_tanh_" + _t: (ci, [vp, vp, ci, ci, vp]),
         "cubert_mean_pool_" + _t: (ci, [vp, vp, ci, ci, ci, vp]),
         "cubert_transpose_" + _t: (ci, [vp, ci, ci, vp, vp]),
+        "cubert_classifier_head_" + _t: (ci, [vp, vp, vp, vp, vp, vp, ci, ci, ci, vp]),
         "cubert_gemm_" + _t: (ci, [vp, ci, ci, ci, ci, ci, cf, vp, ci, vp, ci, cf, vp, ci, vp]),
         "cubert_gemm_skinny_" + _t: (ci, [vp, ci, ci, ci, cf, vp, ci, vp, ci, vp, ci, vp, ci]),
         "cubert_gemm_skinny_pack_" + _t: (ci, [vp, vp, ci, ci, ci, vp]),

@@ -190,22 +190,33 @@ void Bert<T>::forward(size_t batch_size) {
     _sequence_output = transformer->_in_compute(batch_size, _embedding_output, input_mask_buf);
 
     // bert/pooler
+    bool tanh_pending = false;
     if (has_pooler_dense) {
         // first token of every sequence: the B rows are seq_length*hidden apart
-        {
-            Timed t(&profiler, Profiler::kDenseGemm, stream);
-            cuBERT::blas_gemm(cublas, false, false, H, B, H, 1.f, pooler_kernel, H, _sequence_output, H * S, 0.f,
-                              _pooled_output, H);
-        }
-        Timed t(&profiler, Profiler::kBiasTanh, stream);
-        cuBERT::tanh_(_pooled_output, pooler_bias, B, H, stream);
+        Timed t(&profiler, Profiler::kDenseGemm, stream);
+        cuBERT::blas_gemm(cublas, false, false, H, B, H, 1.f, pooler_kernel, H, _sequence_output, H * S, 0.f,
+                          _pooled_output, H);
+        tanh_pending = true;
     } else {
         Timed t(&profiler, Profiler::kMeanPool, stream);
         cuBERT::reduce_mean_1(_sequence_output, _pooled_output, B, S, H, stream);
     }
 
+    // classifier head: pooler bias + tanh, logits = pooled * W^T (+ bias) with W [num_labels, hidden] row-major, and
+    // their softmax -- one launch for few labels, else the three kernels of the reference
+    if (has_classifier && classifier_head_fits) {
+        Timed t(&profiler, Profiler::kClassifierHead, stream);
+        if (cuBERT::classifier_head(_pooled_output, tanh_pending ? pooler_bias : nullptr, output_weights, output_bias,
+                                    _logits, _probs, B, H, L, stream)) {
+            return;
+        }
+        classifier_head_fits = false;  // the sizes are fixed per model: do not ask again
+    }
+    if (tanh_pending) {
+        Timed t(&profiler, Profiler::kBiasTanh, stream);
+        cuBERT::tanh_(_pooled_output, pooler_bias, B, H, stream);
+    }
     if (has_classifier) {
-        // logits = pooled * W^T (+ bias), W is [num_labels, hidden] row-major
         {
             Timed t(&profiler, Profiler::kDenseGemm, stream);
             cuBERT::blas_gemm(cublas, true, false, L, B, H, 1.f, output_weights, H, _pooled_output, H, 0.f, _logits, L,

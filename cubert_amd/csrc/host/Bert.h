@@ -76,6 +76,7 @@ private:
 
     size_t max_batch_size, seq_length, hidden_size, num_labels;
     bool has_pooler_dense, has_classifier, has_classifier_bias;
+    bool classifier_head_fits = true;  // cleared when the one-launch classifier head declines this model's shape
 
     Transformer<T> *transformer = nullptr;
     Profiler profiler;

@@ -25,7 +25,8 @@ public:
         kDenseGemm = 7,
         kAttentionGemm = 8,
         kAttentionFused = 9,
-        kKinds = 10
+        kClassifierHead = 10,
+        kKinds = 11
     };
 
     ~Profiler() {

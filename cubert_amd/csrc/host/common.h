@@ -170,6 +170,25 @@ inline void layer_norm_(const half *in, half *inout, int rows, int channels, con
     CUBERT_CHECK(cubert_bias_res_ln_f16(h(inout), h(in), h(bias), h(beta), h(gamma), rows, channels, stream));
 }
 
+// Pooler bias + tanh (pooler_bias null: none), classifier and its softmax in one launch; false when the kernel
+// does not take the problem (many labels).  reference: op_bert/BertPooler.cpp:65-76, op_out/AdditionalOutputLayer.cpp:52-66
+inline bool classifier_head(float *pooled, const float *pooler_bias, const float *weights, const float *out_bias,
+                            float *logits, float *probs, int batch, int hidden, int labels, void *stream) {
+    const int rc = cubert_classifier_head_f32(pooled, pooler_bias, weights, out_bias, logits, probs, batch, hidden, labels,
+                                              stream);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+inline bool classifier_head(half *pooled, const half *pooler_bias, const half *weights, const half *out_bias,
+                            half *logits, half *probs, int batch, int hidden, int labels, void *stream) {
+    const int rc = cubert_classifier_head_f16(h(pooled), h(pooler_bias), h(weights), h(out_bias), h(logits), h(probs),
+                                              batch, hidden, labels, stream);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+
 // reference: op/GELU.h:6-7, with the Dense bias folded in (bias may be null)
 inline void gelu(float *inout, const float *bias, int rows, int width, void *stream) {
     CUBERT_CHECK(cubert_bias_gelu_f32(inout, bias, rows, width, stream));

@@ -186,6 +186,90 @@ int gather(const Id *ids, int n, const T *table, int width, T *out, void *stream
     return launch(gather_kernel<T, Id, 1>, grid, block, s, ids, n, table, width, out);
 }
 
+// The tail of a classification model in one launch, one workgroup per sequence:
+//   pooled = tanh(pooled + pooler_bias)        (skipped when pooler_bias is null: pooled is final already)
+//   logits = pooled W^T + out_bias             (W [labels, hidden] row-major; out_bias may be null)
+//   probs  = softmax(logits)
+// with few labels these are three launch-bound kernels otherwise (bias + tanh, a GEMM with a handful of output
+// columns, a row softmax).  pooled and logits are rounded to the storage type before they are used further, as
+// the separate kernels store them; the softmax divides by the sum in fp32 and multiplies by its reciprocal in
+// fp16, as cubert_row_softmax_* does.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void classifier_head_kernel(T *__restrict__ pooled, const T *__restrict__ pooler_bias,
+                                                                 const T *__restrict__ weights,
+                                                                 const T *__restrict__ out_bias, T *__restrict__ logits,
+                                                                 T *__restrict__ probs, int hidden, int labels) {
+    extern __shared__ float s_row[];  // [hidden] pooled row, then [labels] logits
+    float *s_logit = s_row + hidden;
+    T *row = pooled + (size_t) blockIdx.x * hidden;
+    const int lane = threadIdx.x & (kWave - 1), wave = wave_in_block();
+    // the weight row of this wavefront's first label is requested before anything else (rows of up to 1024
+    // values; it comes from memory, cold, while the tanh below is computed)
+    constexpr int kAhead = 16;
+    float w_first[kAhead];
+    const bool ahead = wave < labels && hidden <= kAhead * kWave;
+#pragma unroll
+    for (int t = 0; t < kAhead; ++t) {
+        const int j = t * kWave + lane;
+        w_first[t] = ahead && j < hidden ? to_f32(weights[(size_t) wave * hidden + j]) : 0.f;
+    }
+    for (int j = threadIdx.x; j < hidden; j += kBlock) {
+        float v = to_f32(row[j]);
+        if (pooler_bias != nullptr) {
+            const T stored = from_f32<T>(TanhOp()(v + to_f32(pooler_bias[j])));
+            row[j] = stored;
+            v = to_f32(stored);
+        }
+        s_row[j] = v;
+    }
+    __syncthreads();
+    for (int l = wave; l < labels; l += kBlock / kWave) {
+        const T *w = weights + (size_t) l * hidden;
+        float acc = 0.f;
+        if (ahead && l == wave) {
+#pragma unroll
+            for (int t = 0; t < kAhead; ++t) {
+                const int j = t * kWave + lane;
+                acc += j < hidden ? s_row[j] * w_first[t] : 0.f;
+            }
+        } else {
+            for (int j = lane; j < hidden; j += kWave) acc += s_row[j] * to_f32(w[j]);
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) {
+            const T stored = from_f32<T>(acc + (out_bias != nullptr ? to_f32(out_bias[l]) : 0.f));
+            logits[(size_t) blockIdx.x * labels + l] = stored;
+            s_logit[l] = to_f32(stored);
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        float mx = -3.402823466e+38f;
+        for (int l = lane; l < labels; l += kWave) mx = fmaxf(mx, s_logit[l]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int l = lane; l < labels; l += kWave) sum += __expf(s_logit[l] - mx);
+        sum = wave_sum(sum);
+        const float inv = 1.f / sum;
+        for (int l = lane; l < labels; l += kWave) {
+            const float e = __expf(s_logit[l] - mx);
+            probs[(size_t) blockIdx.x * labels + l] = from_f32<T>(sizeof(T) == 4 ? e / sum : e * inv);
+        }
+    }
+}
+
+template <typename T>
+int classifier_head(T *pooled, const T *pooler_bias, const T *weights, const T *out_bias, T *logits, T *probs,
+                    int batch, int hidden, int labels, void *stream) {
+    if (batch < 0 || hidden <= 0 || labels <= 0 || !pooled || !weights || !logits || !probs) return CUBERT_BAD_ARGUMENT;
+    if (batch == 0) return 0;
+    // few labels only: a wavefront walks a whole weight row per label; beyond that a GEMM is the better tool
+    const size_t lds = ((size_t) hidden + labels) * sizeof(float);
+    if (labels > 64 || lds > 48 * 1024) return CUBERT_UNSUPPORTED;
+    return launch_lds(classifier_head_kernel<T>, dim3(batch), dim3(kBlock), (unsigned) lds, (hipStream_t) stream, pooled,
+                      pooler_bias, weights, out_bias, logits, probs, hidden, labels);
+}
+
 // out[c, r] = in[r, c] for a row-major [rows, cols] matrix: 32 x 32 tiles through LDS so that both the reads
 // and the writes are contiguous runs.  Run once per weight matrix when a model is loaded.
 template <typename T>
@@ -258,4 +342,17 @@ extern "C" int cubert_transpose_f32(const float *in, int rows, int cols, float *
 }
 extern "C" int cubert_transpose_f16(const cubert_half *in, int rows, int cols, cubert_half *out, void *stream) {
     return cubert::transpose<half_t>((const half_t *) in, rows, cols, (half_t *) out, stream);
+}
+extern "C" int cubert_classifier_head_f32(float *pooled, const float *pooler_bias, const float *weights,
+                                          const float *out_bias, float *logits, float *probs, int batch, int hidden,
+                                          int labels, void *stream) {
+    return cubert::classifier_head<float>(pooled, pooler_bias, weights, out_bias, logits, probs, batch, hidden, labels,
+                                          stream);
+}
+extern "C" int cubert_classifier_head_f16(cubert_half *pooled, const cubert_half *pooler_bias, const cubert_half *weights,
+                                          const cubert_half *out_bias, cubert_half *logits, cubert_half *probs, int batch,
+                                          int hidden, int labels, void *stream) {
+    return cubert::classifier_head<half_t>((half_t *) pooled, (const half_t *) pooler_bias, (const half_t *) weights,
+                                           (const half_t *) out_bias, (half_t *) logits, (half_t *) probs, batch, hidden,
+                                           labels, stream);
 }

@@ -135,6 +135,22 @@ def mean_pool(x):
     return out
 
 
+def classifier_head_(pooled, pooler_bias, weights, out_bias):
+    """tanh(pooled + pooler_bias) in place (skipped without pooler_bias), logits = pooled W^T + out_bias and their
+    softmax in one launch; returns (logits, probs), or None beyond 64 labels."""
+    batch, hidden = pooled.shape
+    labels = weights.shape[0]
+    logits = torch.empty((batch, labels), dtype=pooled.dtype, device=pooled.device)
+    probs = torch.empty_like(logits)
+    fn = getattr(lib(), "cubert_classifier_head_" + _suffix(pooled))
+    rc = fn(_ptr(pooled), _ptr(pooler_bias), _ptr(weights), _ptr(out_bias), _ptr(logits), _ptr(probs), batch, hidden,
+            labels, _stream())
+    if rc == -2:
+        return None
+    _check(rc, fn.__name__)
+    return logits, probs
+
+
 def transpose(x):
     """The transpose of a row-major 2-D tensor, as a new contiguous tensor."""
     rows, cols = x.shape

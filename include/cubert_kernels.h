@@ -144,6 +144,20 @@ int cubert_mean_pool_f32(const float *in, float *out, int batch, int seq_length,
 int cubert_mean_pool_f16(const cubert_half *in, cubert_half *out, int batch, int seq_length, int hidden,
                          void *stream);
 
+/* The tail of a classification model in one launch (one workgroup per sequence):
+ *     pooled = tanh(pooled + pooler_bias)   in place; skipped when pooler_bias is NULL
+ *     logits = pooled W^T + out_bias        W [labels, hidden] row-major, out_bias may be NULL
+ *     probs  = softmax(logits)
+ * for up to 64 labels (more: CUBERT_UNSUPPORTED, nothing launched; use cubert_bias_tanh_*, cubert_gemm_* and
+ * cubert_row_softmax_*).
+ * replaces: tanh_<T> (op_bert/BertPooler.cpp:65-76), ClassifierOutputLayer<T>::_in_compute and its Softmax<T>
+ * (op_out/AdditionalOutputLayer.cpp:30,52-66). */
+int cubert_classifier_head_f32(float *pooled, const float *pooler_bias, const float *weights, const float *out_bias,
+                               float *logits, float *probs, int batch, int hidden, int labels, void *stream);
+int cubert_classifier_head_f16(cubert_half *pooled, const cubert_half *pooler_bias, const cubert_half *weights,
+                               const cubert_half *out_bias, cubert_half *logits, cubert_half *probs, int batch,
+                               int hidden, int labels, void *stream);
+
 /* out[c, r] = in[r, c] for a row-major [rows, cols] matrix (out must not alias in).  No counterpart in the
  * reference, which keeps every Dense kernel [in, out] (op/Dense.cpp:47-57): half-precision models here store
  * them [out, in], the operand order the library's fp16 GEMMs run fastest on. */

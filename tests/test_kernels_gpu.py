@@ -306,6 +306,49 @@ def test_gather(K, name, idt):
 
 
 @pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("batch,hidden,labels,tanh,bias", [(1, 768, 2, True, True), (128, 768, 2, True, True),
+                                                          (5, 1024, 3, False, True), (7, 100, 1, True, False),
+                                                          (3, 768, 64, True, True)])
+def test_classifier_head(K, name, batch, hidden, labels, tanh, bias):
+    """Pooler bias + tanh, classifier and softmax in one launch against the oracle's tanh_, sgemm (W^T) and
+    softmax_ and against this library's three separate kernels."""
+    rng = np.random.default_rng(batch + hidden + labels)
+    dt = tdt(name)
+    x = q(rng.normal(0, 1, (batch, hidden)), name)
+    pb = q(rng.normal(0, 0.5, hidden), name)
+    W = q(rng.normal(0, 0.1, (labels, hidden)), name)
+    ob = q(rng.normal(0, 1, labels), name) if bias else None
+    pooled = dev(x, dt)
+    out = K.classifier_head_(pooled, dev(pb, dt) if tanh else None, dev(W, dt), None if ob is None else dev(ob, dt))
+    assert out is not None
+    logits, probs = out
+    want_pooled = np.tanh((x + pb[None, :]).astype(np.float32)) if tanh else x
+    if name == "f16":
+        want_pooled = oracle.round_to_half(want_pooled)
+    t = tol(name)
+    assert_close(host(pooled), want_pooled, t, "pooled")
+    want_logits = host(pooled) @ W.T + (0 if ob is None else ob[None, :])
+    if name == "f16":
+        want_logits = oracle.round_to_half(want_logits.astype(np.float32))
+    assert_close(host(logits), want_logits, 2e-5 if name == "f32" else 2e-3, "logits")
+    want_probs = oracle.softmax_(np.ascontiguousarray(host(logits), dtype=np.float32))
+    assert_close(host(probs), want_probs, 2e-5 if name == "f32" else 2e-3, "probs")
+    np.testing.assert_allclose(host(probs).sum(-1), 1.0, atol=1e-5 if name == "f32" else 2e-3)
+    # the three separate kernels
+    p3 = dev(x, dt)
+    if tanh:
+        K.bias_tanh_(p3, dev(pb, dt))
+    assert_close(host(pooled), host(p3), 1e-6 if name == "f32" else 1e-3, "pooled vs bias_tanh")
+    s3 = K.row_softmax(logits)
+    assert_close(host(probs), host(s3), 1e-6 if name == "f32" else 1e-3, "probs vs row_softmax")
+
+
+def test_classifier_head_declines_many_labels(K):
+    z = torch.zeros
+    assert K.classifier_head_(z((2, 64), device="cuda"), None, z((65, 64), device="cuda"), None) is None
+
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
 @pytest.mark.parametrize("rows,cols", [(768, 2304), (3072, 768), (33, 65), (1, 7), (100, 1), (32, 32)])
 def test_transpose(K, name, rows, cols):
     x = q(np.random.default_rng(rows + cols).normal(0, 1, (rows, cols)), name)
