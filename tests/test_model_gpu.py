@@ -89,6 +89,20 @@ def test_small_model_all_outputs_fp32(cb, pooler, bias, scattered):
         assert_close(got[k], want[k], FP32_TOL, k)
 
 
+@pytest.mark.parametrize("compute_type", [0, 1])
+@pytest.mark.parametrize("pooler", [True, False])
+def test_many_labels_take_the_three_kernel_classifier(cb, compute_type, pooler):
+    """More than 64 labels: the one-launch classifier head declines and the model runs bias + tanh, the classifier
+    GEMM and the row softmax separately; with or without a pooler dense layer (MeanPooler)."""
+    from cubert_amd.testing import random_bert_weights, random_inputs
+    w = random_bert_weights(seed=11, labels=70, pooler=pooler, classifier=True, ln_random=True, **SMALL)
+    ids, mask, seg = random_inputs(seed=12, batch=5, seq_length=32, vocab=SMALL["vocab"], min_valid=4, segment_split=11)
+    got, want, _ = run_both(cb, w, ids, mask, seg, 3, 4, max_batch=6, compute_type=compute_type)
+    for k in ("pooled_output", "logits", "probs"):
+        assert_close(got[k], want[k], FP16_TOL if compute_type else FP32_TOL, k)
+    assert got["probs"].shape == (5, 70)
+
+
 def test_small_model_fp16(cb):
     from cubert_amd.testing import random_bert_weights, random_inputs
     w = random_bert_weights(seed=5, labels=2, pooler=True, classifier=True, ln_random=True, **SMALL)
