@@ -304,7 +304,7 @@ class Bert(object):
             raise RuntimeError("stream synchronize failed: %d" % rc)
 
     KINDS = ("embed_ln", "bias_res_ln", "bias_gelu", "mask_scale_softmax", "bias_tanh", "mean_pool", "row_softmax",
-             "dense_gemm", "attention_gemm", "attention_fused", "classifier_head")
+             "dense_gemm", "attention_gemm", "attention_fused", "classifier_head", "dense_split")
 
     def profile(self, kinds):
         """Switch per-kernel event timing on for the named kinds (empty = off)."""

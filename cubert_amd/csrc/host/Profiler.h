@@ -26,7 +26,8 @@ public:
         kAttentionGemm = 8,
         kAttentionFused = 9,
         kClassifierHead = 10,
-        kKinds = 11
+        kDenseSplit = 11,  // fp32 rows written as two-term fp16 rows ahead of a Dense GEMM
+        kKinds = 12
     };
 
     ~Profiler() {

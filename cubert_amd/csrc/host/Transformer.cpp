@@ -44,6 +44,9 @@ Transformer<T>::Transformer(void *cublas, const std::string &var_prefix,
     // 32768 tokens on every Dense shape of BERT-base and BERT-large, same bits out); its fp32 GEMMs do not care.
     // Half-precision models therefore keep their Dense kernels [out, in], transposed once here.
     transposed_kernels = sizeof(T) == 2;
+    const char *dense_mode = std::getenv("CUBERT_FP32_DENSE");
+    split_dense = sizeof(T) == 4 && dense_mode != nullptr && std::string(dense_mode) == "f16x3" &&
+                  max_batch_size * seq_length > 32;
 
     // Weight names as the reference resolves them (Transformer.cpp:54-101, AttentionSelf.cpp:27-44);
     // a missing name throws std::out_of_range from unordered_map::at, as it does there.
@@ -53,16 +56,32 @@ Transformer<T>::Transformer(void *cublas, const std::string &var_prefix,
 
     void *stream = cuBERT::blas_get_stream(cublas);
     const size_t largest = H * (3 * H > I ? 3 * H : I);
-    ScopedDeviceBuffer staging_memory(transposed_kernels ? largest * sizeof(T) : 0);
+    ScopedDeviceBuffer staging_memory(transposed_kernels || split_dense ? largest * sizeof(T) : 0);
     T *staging = static_cast<T *>(staging_memory.ptr);
     // one Dense kernel, [in, out] on the host, into its place on the device (and its few-token copy)
-    auto load_kernel = [&](T *dst, T *few_token_copy, const T *host, size_t in, size_t out) {
+    auto load_kernel = [&](T *dst, T *few_token_copy, SplitKernel &split, const T *host, size_t in, size_t out) {
         T *plain = transposed_kernels ? staging : dst;
         upload(plain, host, in * out);
         if (keep_packed) cuBERT::pack_few_token_weights(cublas, plain, (int) out, (int) out, (int) in, few_token_copy);
         if (transposed_kernels) {
             cuBERT::transpose(plain, (int) in, (int) out, dst, stream);
             cuBERT::cuda_stream_synchronize(stream);  // the staging buffer is written again by the next upload
+        }
+        if constexpr (sizeof(T) == 4) {
+            if (split_dense) {
+                // a power of two that brings the largest weight to [512, 1024): far from fp16's subnormals and its limit
+                float largest_weight = 0.f;
+                for (size_t i = 0; i < in * out; ++i) largest_weight = std::fmax(largest_weight, std::fabs(host[i]));
+                int exponent = 0;
+                if (largest_weight > 0.f && std::isfinite(largest_weight)) {
+                    (void) std::frexp(largest_weight, &exponent);  // largest = f * 2^exponent, f in [0.5, 1)
+                    exponent = 10 - exponent;
+                }
+                split.unscale = std::ldexp(1.f, -exponent);
+                cuBERT::transpose(dst, (int) in, (int) out, staging, stream);
+                cuBERT::split3(staging, (int) out, (int) in, std::ldexp(1.f, exponent), true, split.weights, stream);
+                cuBERT::cuda_stream_synchronize(stream);
+            }
         }
     };
 
@@ -82,16 +101,17 @@ Transformer<T>::Transformer(void *cublas, const std::string &var_prefix,
         std::memcpy(&packed_bias[H], kb, H * sizeof(T));
         std::memcpy(&packed_bias[2 * H], vb, H * sizeof(T));
         Layer &w = layers[l];
-        load_kernel(w.qkv_kernel, w.qkv_packed, packed.data(), H, 3 * H);
+        load_kernel(w.qkv_kernel, w.qkv_packed, w.qkv_split, packed.data(), H, 3 * H);
         upload(w.qkv_bias, packed_bias.data(), 3 * H);
-        load_kernel(w.attention_output_kernel, w.attention_output_packed,
+        load_kernel(w.attention_output_kernel, w.attention_output_packed, w.attention_output_split,
                     var.at(p + "/attention/output/dense/kernel"), H, H);
         upload(w.attention_output_bias, var.at(p + "/attention/output/dense/bias"), H);
         upload(w.attention_norm_beta, var.at(p + "/attention/output/LayerNorm/beta"), H);
         upload(w.attention_norm_gamma, var.at(p + "/attention/output/LayerNorm/gamma"), H);
-        load_kernel(w.intermediate_kernel, w.intermediate_packed, var.at(p + "/intermediate/dense/kernel"), H, I);
+        load_kernel(w.intermediate_kernel, w.intermediate_packed, w.intermediate_split,
+                    var.at(p + "/intermediate/dense/kernel"), H, I);
         upload(w.intermediate_bias, var.at(p + "/intermediate/dense/bias"), I);
-        load_kernel(w.output_kernel, w.output_packed, var.at(p + "/output/dense/kernel"), I, H);
+        load_kernel(w.output_kernel, w.output_packed, w.output_split, var.at(p + "/output/dense/kernel"), I, H);
         upload(w.output_bias, var.at(p + "/output/dense/bias"), H);
         upload(w.output_norm_beta, var.at(p + "/output/LayerNorm/beta"), H);
         upload(w.output_norm_gamma, var.at(p + "/output/LayerNorm/gamma"), H);
@@ -125,6 +145,12 @@ void Transformer<T>::layout_weights() {
             w.intermediate_packed = weights.take<T>(cubert_gemm_skinny_packed_elements((int) I, (int) H));
             w.output_packed = weights.take<T>(cubert_gemm_skinny_packed_elements((int) H, (int) I));
         }
+        if (split_dense) {
+            w.qkv_split.weights = weights.take<half>(3 * H * 3 * H);
+            w.attention_output_split.weights = weights.take<half>(3 * H * H);
+            w.intermediate_split.weights = weights.take<half>(3 * H * I);
+            w.output_split.weights = weights.take<half>(3 * I * H);
+        }
     }
 }
 
@@ -138,6 +164,7 @@ void Transformer<T>::layout_buffers() {
     intermediate_output = buffers.take<T>(M * intermediate_size);
     layer_output[0] = buffers.take<T>(M * H);
     layer_output[1] = buffers.take<T>(M * H);
+    if (split_dense) split_operand = buffers.take<half>(M * 3 * (H > intermediate_size ? H : intermediate_size));
 }
 
 template <typename T>
@@ -234,16 +261,64 @@ bool Transformer<T>::dense(int out_features, int tokens, int in_features, const 
 }
 
 template <typename T>
+void Transformer<T>::dense_split(int out_features, int tokens, int in_features, const SplitKernel &kernel, const T *in,
+                                 T *out, const T *bias) {
+    if constexpr (sizeof(T) == 4) {
+        void *stream = cuBERT::blas_get_stream(cublas);
+        if (in != nullptr) {
+            Timed t(profiler, Profiler::kDenseSplit, stream);
+            cuBERT::split3(in, tokens, in_features, 1.f, false, split_operand, stream);
+        }
+        Timed t(profiler, Profiler::kDenseGemm, stream);
+        cuBERT::blas_gemm_f16_f32(cublas, true, false, out_features, tokens, 3 * in_features, kernel.unscale,
+                                  kernel.weights, 3 * in_features, split_operand, 3 * in_features, 0.f, out,
+                                  out_features, bias);
+    } else {
+        throw std::logic_error("the two-term fp16 Dense form is for fp32 models");
+    }
+}
+
+template <typename T>
 T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attention_mask) {
     if (batch_size > max_batch_size) throw std::invalid_argument("batch_size > max_batch_size");
     void *stream = cuBERT::blas_get_stream(cublas);
     const int M = (int) (batch_size * seq_length), H = (int) hidden_size, I = (int) intermediate_size;
+
+    // (requests of at most 32 tokens are one pass over the weights whatever the arithmetic: they keep the fp32 kernels)
+    const bool split = split_dense && M > 32;
 
     T *prev_output = input_gpu;
     for (size_t l = 0; l < num_hidden_layers; ++l) {
         const Layer &w = layers[l];
         T *layer_input = prev_output;
         T *out = layer_output[l & 1];
+
+        if (split) {
+            dense_split(3 * H, M, H, w.qkv_split, layer_input, qkv_out, w.qkv_bias);
+            attention(batch_size, qkv_out, attention_mask);
+            dense_split(H, M, H, w.attention_output_split, context_out, attention_output, nullptr);
+            {
+                Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
+                cuBERT::layer_norm_(layer_input, attention_output, M, H, w.attention_output_bias, w.attention_norm_beta,
+                                    w.attention_norm_gamma, stream);
+            }
+            dense_split(I, M, H, w.intermediate_split, attention_output, intermediate_output, nullptr);
+            {
+                // bias + GELU straight into the two-term rows the output Dense reads
+                Timed t(profiler, Profiler::kBiasGelu, stream);
+                if constexpr (sizeof(T) == 4) {
+                    cuBERT::bias_gelu_split3(intermediate_output, w.intermediate_bias, M, I, split_operand, stream);
+                }
+            }
+            dense_split(H, M, I, w.output_split, nullptr, out, nullptr);
+            {
+                Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
+                cuBERT::layer_norm_(attention_output, out, M, H, w.output_bias, w.output_norm_beta, w.output_norm_gamma,
+                                    stream);
+            }
+            prev_output = out;
+            continue;
+        }
 
         // attention/self: row-major Y[M, N] = X[M, K] W[K, N] is the column-major gemm(N, M, K) on (W, X)
         dense(3 * H, M, H, w.qkv_kernel, w.qkv_packed, layer_input, qkv_out, w.qkv_bias, true, false);

@@ -15,6 +15,12 @@
 // Activation buffers are shared by all layers (the reference keeps four private
 // buffers per layer); weights live in one device allocation.  A half-precision model whose seq_length allows
 // requests of at most 32 tokens also keeps its four Dense kernels in the few-token GEMM kernel's own order.
+//
+// CUBERT_FP32_DENSE=f16x3 in the environment when an fp32 model is opened makes its Dense layers of more than 32
+// tokens run on the fp16 matrix cores: every fp32 operand is written as the sum of two fp16 numbers and the
+// product as hi*hi + hi*lo + lo*hi with fp32 accumulation (one GEMM over three times the reduction length), which
+// keeps the error of an fp32 GEMM for activations inside the fp16 range (|x| <= 65504; see kernels/split.hip).
+// Everything between the GEMMs stays fp32.  The default is the fp32 GEMM.
 #ifndef CUBERT_HOST_TRANSFORMER_H
 #define CUBERT_HOST_TRANSFORMER_H
 
@@ -25,6 +31,7 @@
 #include <vector>
 
 #include "Arena.h"
+#include "common.h"
 #include "Profiler.h"
 
 namespace cuBERT {
@@ -51,6 +58,12 @@ public:
     void set_profiler(Profiler *p) { profiler = p; }
 
 private:
+    // A Dense kernel for the two-term fp16 form: rows [hi | lo | hi] of scale * W^T, [out, 3 * in]; unscale = 1 / scale
+    struct SplitKernel {
+        half *weights = nullptr;
+        float unscale = 1.f;
+    };
+
     struct Layer {
         // Dense kernels are [in, out] as in the model file, or [out, in] when transposed_kernels is set
         T *qkv_kernel, *qkv_bias;            // [hidden, 3*hidden] (query | key | value side by side), [3*hidden]
@@ -62,6 +75,7 @@ private:
         // the Dense kernels again, in the few-token GEMM kernel's order (null when not kept)
         T *qkv_packed = nullptr, *attention_output_packed = nullptr, *intermediate_packed = nullptr,
           *output_packed = nullptr;
+        SplitKernel qkv_split, attention_output_split, intermediate_split, output_split;  // (null when not kept)
     };
 
     void layout_weights();
@@ -71,12 +85,17 @@ private:
     // activation were applied (false: the caller's fused kernel still has to).
     bool dense(int out_features, int tokens, int in_features, const T *kernel, const T *packed, const T *in, T *out,
                const T *bias, bool bias_in_gemm, bool gelu);
+    // The same on the fp16 matrix cores from two-term operands (fp32 models only): `in` is split into
+    // split_operand first, or, when null, split_operand already holds the [hi | hi | lo] rows.  `bias` may be null.
+    void dense_split(int out_features, int tokens, int in_features, const SplitKernel &kernel, const T *in, T *out,
+                     const T *bias);
 
     void *cublas;
     Profiler *profiler = nullptr;
     bool dense_gelu_fits = true;       // cleared when the few-token Dense + GELU kernel declines this model's shape
     bool keep_packed = false;          // Dense kernels are also kept in the few-token kernel's order
     bool transposed_kernels = false;   // Dense kernels are stored [out, in] instead of [in, out] (half precision)
+    bool split_dense = false;          // fp32 model with Dense layers in the two-term fp16 form (opt-in)
     bool fused_attention_fits = true;  // cleared when the one-launch attention kernel declines this model's shape
     size_t max_batch_size, seq_length, hidden_size, num_hidden_layers, num_attention_heads, intermediate_size;
 
@@ -90,6 +109,7 @@ private:
     T *attention_output;     // [M, hidden]
     T *intermediate_output;  // [M, intermediate]
     T *layer_output[2];      // [M, hidden], alternating between layers
+    half *split_operand = nullptr;  // [M, 3 * max(hidden, intermediate)] two-term rows of the current Dense input
 };
 
 }  // namespace cuBERT

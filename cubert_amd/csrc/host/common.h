@@ -109,6 +109,19 @@ inline void pack_few_token_weights(void *handle, const half *A, int lda, int M, 
     CUBERT_CHECK(cubert_gemm_skinny_pack_f16(handle, h(A), lda, M, K, h(packed)));
 }
 
+// fp16 operands, fp32 result: the Dense GEMM of an fp32 model in its two-term fp16 form (kernels/split.hip)
+inline void blas_gemm_f16_f32(void *handle, bool TransA, bool TransB, int M, int N, int K, float alpha, const half *A,
+                              int lda, const half *B, int ldb, float beta, float *C, int ldc,
+                              const float *bias = nullptr) {
+    CUBERT_CHECK(cubert_gemm_f16_f32(handle, TransA, TransB, M, N, K, alpha, h(A), lda, h(B), ldb, beta, C, ldc, bias));
+}
+inline void split3(const float *in, int rows, int width, float scale, bool lo_in_middle, half *out, void *stream) {
+    CUBERT_CHECK(cubert_split3_f32(in, rows, width, scale, lo_in_middle, h(out), stream));
+}
+inline void bias_gelu_split3(const float *in, const float *bias, int rows, int width, half *out, void *stream) {
+    CUBERT_CHECK(cubert_bias_gelu_split3_f32(in, bias, rows, width, h(out), stream));
+}
+
 inline void transpose(const float *in, int rows, int cols, float *out, void *stream) {
     CUBERT_CHECK(cubert_transpose_f32(in, rows, cols, out, stream));
 }

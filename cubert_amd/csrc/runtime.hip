@@ -58,7 +58,7 @@ constexpr size_t kSkinnyPartialFloats = 1u << 20;
 constexpr int kSkinnyCounters = 4096;
 
 struct GemmKey {
-    int type;  // 0 = f32, 1 = f16
+    int type;  // 0 = f32, 1 = f16, 2 = f16 operands with an f32 result
     int transA, transB, M, N, K, lda, ldb, ldc, batch;
     long long strideA, strideB, strideC;
     bool bias;
@@ -114,7 +114,8 @@ int make_layout(hipblasLtMatrixLayout_t *out, hipDataType type, int rows, int co
 }
 
 int build_plan(BlasContext *ctx, const GemmKey &k, GemmPlan *plan) {
-    const hipDataType type = k.type == 0 ? HIP_R_32F : HIP_R_16F;
+    const hipDataType type = k.type == 0 ? HIP_R_32F : HIP_R_16F;        // of A and B
+    const hipDataType out_type = k.type == 1 ? HIP_R_16F : HIP_R_32F;    // of C and the bias
     LT_TRY(hipblasLtMatmulDescCreate(&plan->desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
     hipblasOperation_t ta = k.transA ? HIPBLAS_OP_T : HIPBLAS_OP_N, tb = k.transB ? HIPBLAS_OP_T : HIPBLAS_OP_N;
     LT_TRY(hipblasLtMatmulDescSetAttribute(plan->desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof ta));
@@ -122,7 +123,7 @@ int build_plan(BlasContext *ctx, const GemmKey &k, GemmPlan *plan) {
     if (k.bias) {
         hipblasLtEpilogue_t ep = HIPBLASLT_EPILOGUE_BIAS;
         LT_TRY(hipblasLtMatmulDescSetAttribute(plan->desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &ep, sizeof ep));
-        int32_t bt = (int32_t) type;
+        int32_t bt = (int32_t) out_type;
         LT_TRY(hipblasLtMatmulDescSetAttribute(plan->desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bt, sizeof bt));
         // the heuristic wants a bias pointer to be present; the real one is set per call
         const void *dummy = ctx->workspace;
@@ -131,7 +132,7 @@ int build_plan(BlasContext *ctx, const GemmKey &k, GemmPlan *plan) {
     int rc;
     if ((rc = make_layout(&plan->a, type, k.transA ? k.K : k.M, k.transA ? k.M : k.K, k.lda, k.batch, k.strideA))) return rc;
     if ((rc = make_layout(&plan->b, type, k.transB ? k.N : k.K, k.transB ? k.K : k.N, k.ldb, k.batch, k.strideB))) return rc;
-    if ((rc = make_layout(&plan->c, type, k.M, k.N, k.ldc, k.batch, k.strideC))) return rc;
+    if ((rc = make_layout(&plan->c, out_type, k.M, k.N, k.ldc, k.batch, k.strideC))) return rc;
 
     hipblasLtMatmulPreference_t pref;
     LT_TRY(hipblasLtMatmulPreferenceCreate(&pref));
@@ -259,18 +260,18 @@ void tune_plan(BlasContext *ctx, const GemmKey &k, GemmPlan &p, float alpha, con
 // Plain one-thread-per-output GEMM (fp32 accumulation, k ascending).  Used for shapes hipBLASLt has no
 // algorithm for (tiny or oddly aligned operands) and, with CUBERT_GEMM=naive in the environment, for all
 // of them, which gives an independent check of the hipBLASLt call convention.
-template <typename T>
+template <typename T, typename TC = T>
 __global__ void naive_gemm_kernel(int transA, int transB, int M, int N, int K, float alpha, const T *__restrict__ A,
                                   int lda, long long strideA, const T *__restrict__ B, int ldb, long long strideB,
-                                  float beta, T *__restrict__ C, int ldc, long long strideC, int batch,
-                                  const T *__restrict__ bias) {
+                                  float beta, TC *__restrict__ C, int ldc, long long strideC, int batch,
+                                  const TC *__restrict__ bias) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     const int j = blockIdx.y * blockDim.y + threadIdx.y;
     if (i >= M || j >= N) return;
     for (int z = blockIdx.z; z < batch; z += gridDim.z) {
         const T *a = A + z * strideA;
         const T *b = B + z * strideB;
-        T *c = C + z * strideC;
+        TC *c = C + z * strideC;
         float acc = 0.f;
         for (int k = 0; k < K; ++k) {
             const float av = (float) (transA ? a[k + (size_t) i * lda] : a[i + (size_t) k * lda]);
@@ -280,7 +281,7 @@ __global__ void naive_gemm_kernel(int transA, int transB, int M, int N, int K, f
         float v = alpha * acc;
         if (beta != 0.f) v += beta * (float) c[i + (size_t) j * ldc];
         if (bias != nullptr) v += (float) bias[i];
-        c[i + (size_t) j * ldc] = (T) v;
+        c[i + (size_t) j * ldc] = (TC) v;
     }
 }
 
@@ -293,10 +294,14 @@ int run_naive_gemm(hipStream_t stream, int type, int transA, int transB, int M, 
         hipLaunchKernelGGL(naive_gemm_kernel<float>, grid, block, 0, stream, transA, transB, M, N, K, alpha,
                            (const float *) A, lda, strideA, (const float *) B, ldb, strideB, beta, (float *) C, ldc,
                            strideC, batch, (const float *) bias);
-    } else {
+    } else if (type == 1) {
         hipLaunchKernelGGL(naive_gemm_kernel<_Float16>, grid, block, 0, stream, transA, transB, M, N, K, alpha,
                            (const _Float16 *) A, lda, strideA, (const _Float16 *) B, ldb, strideB, beta,
                            (_Float16 *) C, ldc, strideC, batch, (const _Float16 *) bias);
+    } else {
+        hipLaunchKernelGGL((naive_gemm_kernel<_Float16, float>), grid, block, 0, stream, transA, transB, M, N, K, alpha,
+                           (const _Float16 *) A, lda, strideA, (const _Float16 *) B, ldb, strideB, beta, (float *) C,
+                           ldc, strideC, batch, (const float *) bias);
     }
     return hip_rc(hipGetLastError());
 }
@@ -343,7 +348,7 @@ int run_gemm(void *handle, int type, int transA, int transB, int M, int N, int K
         return run_naive_gemm(ctx->stream, type, transA, transB, M, N, K, alpha, A, lda, strideA, B, ldb, strideB,
                               beta, C, ldc, strideC, batch, bias);
     }
-    if (!transA && !transB && batch == 1 && beta == 0.f && N <= 32 && !library_gemm_only()) {
+    if (type != 2 && !transA && !transB && batch == 1 && beta == 0.f && N <= 32 && !library_gemm_only()) {
         const int rc = run_skinny(ctx, type, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, 0);
         if (rc != CUBERT_UNSUPPORTED) return rc;
     }
@@ -522,6 +527,11 @@ int cubert_gemm_f16(void *handle, int transA, int transB, int M, int N, int K, f
                     int lda, const cubert_half *B, int ldb, float beta, cubert_half *C, int ldc,
                     const cubert_half *bias) {
     return run_gemm(handle, 1, transA, transB, M, N, K, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc, 0, 1, bias);
+}
+
+int cubert_gemm_f16_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha, const cubert_half *A,
+                        int lda, const cubert_half *B, int ldb, float beta, float *C, int ldc, const float *bias) {
+    return run_gemm(handle, 2, transA, transB, M, N, K, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc, 0, 1, bias);
 }
 
 int cubert_gemm_skinny_f32(void *handle, int M, int N, int K, float alpha, const float *A, int lda, const float *B,

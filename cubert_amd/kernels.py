@@ -151,6 +151,24 @@ def classifier_head_(pooled, pooler_bias, weights, out_bias):
     return logits, probs
 
 
+def split3(x, scale=1.0, lo_in_middle=False):
+    """fp32 rows [rows, width] as fp16 rows [rows, 3 * width]: hi | hi | lo (lo_in_middle: hi | lo | hi)."""
+    rows, width = x.shape
+    out = torch.empty((rows, 3 * width), dtype=torch.float16, device=x.device)
+    _check(lib().cubert_split3_f32(_ptr(x), rows, width, float(scale), int(lo_in_middle), _ptr(out), _stream()),
+           "cubert_split3_f32")
+    return out
+
+
+def bias_gelu_split3(x, bias):
+    """GELU(x + bias) of fp32 rows as fp16 rows [rows, 3 * width]: hi | hi | lo."""
+    rows, width = x.shape
+    out = torch.empty((rows, 3 * width), dtype=torch.float16, device=x.device)
+    _check(lib().cubert_bias_gelu_split3_f32(_ptr(x), _ptr(bias), rows, width, _ptr(out), _stream()),
+           "cubert_bias_gelu_split3_f32")
+    return out
+
+
 def transpose(x):
     """The transpose of a row-major 2-D tensor, as a new contiguous tensor."""
     rows, cols = x.shape
@@ -183,6 +201,12 @@ class Blas(object):
         """Column-major C = alpha op(A) op(B) + beta C (+ bias per row of C) on flat tensors."""
         _call("cubert_gemm", C, self.handle, int(transA), int(transB), M, N, K, float(alpha), _ptr(A), lda, _ptr(B),
               ldb, float(beta), _ptr(C), ldc, _ptr(bias))
+        return C
+
+    def gemm_f16_f32(self, transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, bias=None):
+        """The same with fp16 A and B and fp32 C and bias."""
+        _check(lib().cubert_gemm_f16_f32(self.handle, int(transA), int(transB), M, N, K, float(alpha), _ptr(A), lda,
+                                         _ptr(B), ldb, float(beta), _ptr(C), ldc, _ptr(bias)), "cubert_gemm_f16_f32")
         return C
 
     def gemm_skinny(self, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias=None, gelu=False):

@@ -214,6 +214,29 @@ int cubert_gemm_f32(void *handle, int transA, int transB, int M, int N, int K, f
 int cubert_gemm_f16(void *handle, int transA, int transB, int M, int N, int K, float alpha,
                     const cubert_half *A, int lda, const cubert_half *B, int ldb, float beta, cubert_half *C,
                     int ldc, const cubert_half *bias);
+/* The same with fp16 operands and an fp32 result (C and bias are float; the products are exact and accumulate in
+ * fp32).  With operands written by cubert_split3_f32 this is the Dense GEMM of an fp32 model on the fp16 matrix
+ * cores.  replaces: blas_gemm<float>, reference src/cuBERT/common.h:59-68 (common.cpp:224-258), as an opt-in
+ * alternative to cubert_gemm_f32. */
+int cubert_gemm_f16_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha,
+                        const cubert_half *A, int lda, const cubert_half *B, int ldb, float beta, float *C, int ldc,
+                        const float *bias);
+
+/* fp32 rows as sums of two fp16 numbers: with hi = fp16(scale * x) and lo = fp16(scale * x - hi),
+ *   out[r] = [hi(in[r]) | hi(in[r]) | lo(in[r])]      (lo_in_middle = 0: the token side of a Dense GEMM)
+ *   out[r] = [hi(in[r]) | lo(in[r]) | hi(in[r])]      (lo_in_middle = 1: the weight side, rows = output features)
+ * each part `width` halves, so that a dot product of a token row with a weight row over 3 * width is
+ * hi*hi + hi*lo + lo*hi = the fp32 product up to 2^-22 relative.  Values are clamped to the fp16 range; `scale`
+ * (a power of two, undone by the GEMM's alpha) keeps small weights out of the fp16 subnormals.
+ * replaces: nothing in the reference by itself; it is the operand preparation of the opt-in form of
+ * Dense<float>::compute (reference src/cuBERT/op/Dense.cpp:47-57) that runs on the fp16 matrix cores. */
+int cubert_split3_f32(const float *in, int rows, int width, float scale, int lo_in_middle, cubert_half *out,
+                      void *stream);
+/* bias + GELU as cubert_bias_gelu_f32 computes it, written as [hi | hi | lo] rows for the GEMM that follows
+ * instead of in place.  replaces: gelu<float>, reference src/cuBERT/op/GELU.h:6-7 (op/GELU.cu:14-26), followed
+ * by the operand preparation above. */
+int cubert_bias_gelu_split3_f32(const float *in, const float *bias, int rows, int width, cubert_half *out,
+                                void *stream);
 
 /* C = alpha * A * B + bias for N <= 32 columns (no transposes, beta = 0): the Dense layer of a request with at
  * most 32 tokens, where A is the [in, out] weight matrix (M = out, K = in) and each column of B one token.
