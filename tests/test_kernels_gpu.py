@@ -356,6 +356,90 @@ def test_transpose(K, name, rows, cols):
     assert got.shape == (cols, rows) and np.array_equal(got, x.T)  # a copy: bit exact
 
 
+# ------------------------------------------------------------------ fp32 Dense on the fp16 matrix cores (opt-in form)
+
+def two_terms(x):
+    """numpy's statement of the split: hi = fp16(x), lo = fp16(x - hi), both round-to-nearest-even."""
+    x = np.asarray(x, np.float32)
+    hi = x.astype(np.float16)
+    lo = (x - hi.astype(np.float32)).astype(np.float16)
+    return hi, lo
+
+
+@pytest.mark.parametrize("rows,width", [(64, 768), (33, 3072), (5, 24), (3, 7), (1, 1), (16, 8)])
+@pytest.mark.parametrize("lo_in_middle", [False, True])
+def test_split3_bit_exact(K, rows, width, lo_in_middle):
+    rng = np.random.default_rng(rows * 7 + width)
+    x = rng.normal(0, 1, (rows, width)).astype(np.float32)
+    x.flat[::5] *= 1e-4   # lo parts in the fp16 subnormals
+    x.flat[::7] *= 300.0
+    x.flat[0] = 70000.0   # beyond fp16: hi saturates at 65504, lo carries the rest
+    scale = 4.0
+    got = K.split3(dev(x), scale, lo_in_middle)
+    torch.cuda.synchronize()
+    got = got.cpu().numpy()
+    clipped = np.clip(x * np.float32(scale), -65504, 65504)
+    hi = clipped.astype(np.float16)
+    lo = np.clip(x * np.float32(scale) - hi.astype(np.float32), -65504, 65504).astype(np.float16)
+    parts = [hi, lo, hi] if lo_in_middle else [hi, hi, lo]
+    assert got.dtype == np.float16 and got.shape == (rows, 3 * width)
+    for i, part in enumerate(parts):
+        assert np.array_equal(got[:, i * width:(i + 1) * width].view(np.uint16), part.view(np.uint16)), i
+    # the two terms carry the value to 2^-22 relative (2^-25 absolute once lo is subnormal)
+    back = hi.astype(np.float64) + lo.astype(np.float64)
+    want = (x * np.float32(scale)).astype(np.float64)
+    ok = np.abs(want) <= 65504
+    assert np.all(np.abs(back - want)[ok] <= np.maximum(np.abs(want)[ok] * 2.0 ** -22, 2.0 ** -25))
+
+
+@pytest.mark.parametrize("rows,width", [(40, 3072), (7, 512), (3, 20), (2, 5)])
+def test_bias_gelu_split3_against_oracle(K, rows, width):
+    rng = np.random.default_rng(width)
+    x = (rng.normal(0, 2, (rows, width))).astype(np.float32)
+    b = rng.normal(0, 0.5, width).astype(np.float32)
+    got = K.bias_gelu_split3(dev(x), dev(b))
+    torch.cuda.synchronize()
+    got = got.cpu().numpy()
+    assert np.array_equal(got[:, :width].view(np.uint16), got[:, width:2 * width].view(np.uint16))
+    value = got[:, :width].astype(np.float64) + got[:, 2 * width:].astype(np.float64)
+    want = oracle.gelu(x + b)
+    assert_close(value, want, FP32_TOL, "two-term GELU")
+    # and against the in-place kernel, to the resolution of the two terms
+    inplace = host(K.bias_gelu_(dev(x), dev(b))).astype(np.float64)
+    assert np.all(np.abs(value - inplace) <= np.maximum(np.abs(inplace) * 2.0 ** -21, 2.0 ** -24))
+
+
+@pytest.mark.parametrize("tokens,in_features,out_features", [(4096, 768, 2304), (200, 3072, 768), (64, 128, 512),
+                                                             (33, 40, 24)])
+def test_two_term_dense_matches_fp32_dense(K, tokens, in_features, out_features):
+    """Dense(x) = x W + b with both operands in two-term fp16 form on the mixed GEMM, against float64 and against
+    the fp32 GEMM: the error of the form is that of fp32 arithmetic (accumulation rounding dominates both)."""
+    rng = np.random.default_rng(tokens + in_features)
+    x = rng.normal(0, 1, (tokens, in_features)).astype(np.float32)
+    w = rng.normal(0, 0.02, (in_features, out_features)).astype(np.float32)
+    b = rng.normal(0, 0.02, out_features).astype(np.float32)
+    want = x.astype(np.float64) @ w.astype(np.float64) + b
+    blas = K.Blas()
+    dx, dw, db = dev(x), dev(w), dev(b)
+    plain = torch.empty((tokens, out_features), dtype=torch.float32, device="cuda")
+    blas.gemm(False, False, out_features, tokens, in_features, 1.0, dw, out_features, dx, in_features, 0.0, plain,
+              out_features, db)
+    exponent = 10 - math.frexp(float(np.abs(w).max()))[1]
+    w3 = K.split3(K.transpose(dw), 2.0 ** exponent, True)       # [out, 3 in]: hi | lo | hi
+    x3 = K.split3(dx)                                           # [tokens, 3 in]: hi | hi | lo
+    out = torch.empty((tokens, out_features), dtype=torch.float32, device="cuda")
+    blas.gemm_f16_f32(True, False, out_features, tokens, 3 * in_features, 2.0 ** -exponent, w3, 3 * in_features, x3,
+                      3 * in_features, 0.0, out, out_features, db)
+    plain, out = host(plain), host(out)
+    blas.close()
+    err_plain = np.linalg.norm(plain - want) / np.linalg.norm(want)
+    err_two_term = np.linalg.norm(out - want) / np.linalg.norm(want)
+    print("\nrelative error vs float64: fp32 GEMM %.2e, two-term fp16 GEMM %.2e" % (err_plain, err_two_term))
+    assert err_two_term < 2e-6
+    assert err_two_term < 2 * err_plain + 2e-7
+    assert_close(out, plain, FP32_TOL, "two-term Dense vs fp32 Dense")
+
+
 # ------------------------------------------------------------------ attention contractions (matrix-core kernels)
 
 @pytest.mark.parametrize("name", ["f32", "f16"])

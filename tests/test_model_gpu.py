@@ -198,6 +198,41 @@ def test_benchmark_configurations(cb, name, rows):
     np.testing.assert_allclose(seq.var(-1), 1.0, atol=1e-2 if half else 1e-4)
 
 
+def test_two_term_fp16_dense_of_an_fp32_model(cb, monkeypatch):
+    """CUBERT_FP32_DENSE=f16x3 (read when a model is opened): the Dense layers of an fp32 model on the fp16 matrix
+    cores from two-term operands.  Same bound as the default path, 1e-5 of the oracle, at the full C1 shape and on a
+    small model with a scattered mask, random LayerNorm weights and more than 32 tokens; requests of at most 32
+    tokens keep the fp32 kernels."""
+    from cubert_amd.testing import CONFIGS, config_inputs, config_weights, random_bert_weights, random_inputs
+    monkeypatch.setenv("CUBERT_FP32_DENSE", "f16x3")
+    cfg = CONFIGS["C1"]
+    m = cfg["model"]
+    w = config_weights("C1", seed=0)
+    ids, mask, seg = config_inputs("C1", seed=0)
+    bert = cb.Bert(w, cfg["batch"], cfg["seq_length"], m["layers"], m["heads"], 0)
+    bert.profile(["dense_split", "dense_gemm"])
+    got = bert.forward(ids, mask, seg)
+    counts = bert.profile_read()
+    assert counts["dense_split"][1] == 3 * m["layers"], counts   # the form was in use
+    one = bert.forward(ids[:1], mask[:1], seg[:1])               # 32 tokens: fp32 few-token kernels
+    assert "dense_split" not in bert.profile_read()
+    bert.close()
+    want = oracle.bert_forward(w, ids, mask, seg, m["layers"], m["heads"])
+    report = {}
+    for k in ("pooled_output", "logits", "probs", "sequence_output", "embedding_output"):
+        report[k] = assert_close(got[k], want[k], FP32_TOL, "C1 two-term " + k)
+        assert_close(one[k], want[k][:1], FP32_TOL, "C1 single request " + k)
+    print("\nC1 two-term Dense, relative errors vs oracle: %s" % {k: "%.2e" % v for k, v in report.items()})
+
+    w = random_bert_weights(seed=3, labels=3, pooler=True, classifier=True, classifier_bias=True, ln_random=True,
+                            **SMALL)
+    ids, mask, seg = random_inputs(seed=4, batch=7, seq_length=32, vocab=SMALL["vocab"], min_valid=2,
+                                   segment_split="random", scattered_mask=True)
+    got, want, _ = run_both(cb, w, ids, mask, seg, 3, 4, max_batch=9)
+    for k in ("embedding_output", "sequence_output", "pooled_output", "logits", "probs"):
+        assert_close(got[k], want[k], FP32_TOL, "small two-term " + k)
+
+
 def test_sequences_of_a_batch_are_independent_at_full_size(cb):
     """A size-independent property at a benchmark shape (C2: fp16, batch 32 x seq 128, heavy padding): permuting the
     sequences of a batch permutes the outputs, and a sequence computed alone gives what it gives inside the batch."""
