@@ -52,8 +52,29 @@ MEASURED_TRAFFIC = {
 }
 
 
+def two_term_dense():
+    """CUBERT_FP32_DENSE=f16x3 in the environment: fp32 models run their Dense layers of more than 32 tokens on the
+    fp16 matrix cores from two-term operands (opt-in; the default is the fp32 GEMM)."""
+    return os.environ.get("CUBERT_FP32_DENSE") == "f16x3"
+
+
 def algorithmic_bytes(cfg):
     """Minimum HBM traffic per launch of each fused kernel (bytes): every operand once."""
+    m = cfg["model"]
+    B, S = cfg["batch"], cfg["seq_length"]
+    H, I, A = m["hidden"], m["intermediate"], m["heads"]
+    e = 4 if cfg["dtype"] == "f32" else 2
+    M = B * S
+    if two_term_dense() and e == 4 and M > 32:
+        # bias+GELU reads fp32 and writes [hi | hi | lo] fp16 rows; the LayerNorm writes both forms
+        extra = {"bias_gelu": M * I * (4 + 6) + I * 4, "bias_res_ln": 3 * M * H * 4 + 3 * H * 4 + 6 * M * H,
+                 "dense_split": M * H * (4 + 6)}
+    else:
+        extra = {}
+    return dict(_algorithmic_bytes(cfg), **extra)
+
+
+def _algorithmic_bytes(cfg):
     m = cfg["model"]
     B, S = cfg["batch"], cfg["seq_length"]
     H, I, A = m["hidden"], m["intermediate"], m["heads"]
@@ -144,6 +165,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="instead of the model: 10 launches of a plain row copy of known size (100 MB read, 100 MB "
                          "written), the yardstick for hardware traffic counters")
+    ap.add_argument("--no-two-term", action="store_true",
+                    help="skip the extra leg that repeats the steps with CUBERT_FP32_DENSE=f16x3 (fp32 workloads)")
     ap.add_argument("--device-only", action="store_true",
                     help="only the device-resident steps (no host-path / batch-1 latency loops): for profiler runs")
     args = ap.parse_args()
@@ -197,7 +220,7 @@ def main():
     value = B / (ms_per_step * 1e-3)
 
     alg = algorithmic_bytes(cfg)
-    traffic = MEASURED_TRAFFIC.get(args.workload, {}).get(dominant)
+    traffic = None if two_term_dense() else MEASURED_TRAFFIC.get(args.workload, {}).get(dominant)
     if dominant in prof:
         total_ms, launches = prof[dominant]
         avg_us = total_ms * 1e3 / launches
@@ -253,6 +276,29 @@ def main():
         p50_b1 = round(float(np.median(lat1)), 3)
     bert.close()
 
+    # ---- the same steps with the opt-in two-term fp16 Dense form of fp32 models (reported beside `value`, never as it)
+    two_term = None
+    if not half and B * S > 32 and not two_term_dense() and not args.device_only and not args.no_two_term:
+        os.environ["CUBERT_FP32_DENSE"] = "f16x3"  # read when a model is opened
+        try:
+            other = cubert_amd.Bert(w, B, S, m["layers"], m["heads"], 0)
+        finally:
+            del os.environ["CUBERT_FP32_DENSE"]
+        other.compute(ids, mask, seg)
+        other.synchronize()
+        for _ in range(args.warmup):
+            other.compute_resident(B)
+        other.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            other.compute_resident(B)
+        other.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        other.close()
+        two_term = {"value": round(B / (ms * 1e-3), 1), "unit": "sequences/s", "ms_per_step": round(ms, 4),
+                    "dtype": "f32 storage and accumulation; Dense products as three f16 matrix-core products of two-term "
+                             "operands (CUBERT_FP32_DENSE=f16x3, opt-in)"}
+
     # ---- CPU baseline: the oracle (a port of the reference's CPU path) on this host's cores
     cpu = None
     if not args.no_cpu and not args.device_only:
@@ -304,6 +350,10 @@ def main():
         "roofline": roofline, "cpu_baseline": cpu,
         "p50_ms_batch1_host_path": p50_b1, "host_path": host_path,
     }
+    if two_term_dense() and not half:
+        line["dtype"] = "f32 storage and accumulation; Dense products as three f16 matrix-core products of two-term operands"
+    if two_term is not None:
+        line["two_term_fp16_dense"] = two_term
     if kernels:
         line["kernels"] = kernels
     print(json.dumps(line))

@@ -182,7 +182,7 @@ void Transformer<T>::_pre_compute(size_t) {}
 // problems have two strides (b: seq*3H, a: d), a strided-batched GEMM has one, so the shorter of the two
 // axes is looped on the host and the longer one is the GEMM batch.
 template <typename T>
-void Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *mask) {
+bool Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *mask, half *split_context) {
     void *stream = cuBERT::blas_get_stream(cublas);
     const int S = (int) seq_length, A = (int) num_attention_heads, H = (int) hidden_size, d = H / A;
     const int B = (int) batch_size, ld = 3 * H;
@@ -200,7 +200,13 @@ void Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *ma
     }();
     if (!split_only && fused_attention_fits) {
         Timed t(profiler, Profiler::kAttentionFused, stream);
-        if (cuBERT::attention_fused(Q, K, V, ld, mask, context_out, H, alpha, B, A, S, d, stream)) return;
+        if constexpr (sizeof(T) == 4) {
+            if (split_context != nullptr &&
+                cuBERT::attention_fused_split3(Q, K, V, ld, mask, split_context, alpha, B, A, S, d, stream)) {
+                return true;
+            }
+        }
+        if (cuBERT::attention_fused(Q, K, V, ld, mask, context_out, H, alpha, B, A, S, d, stream)) return false;
         fused_attention_fits = false;  // seq_length and head size are fixed per model: do not ask again
     }
 
@@ -235,6 +241,7 @@ void Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *ma
                                             context_out + o * ctx_outer, H, ctx_inner, inner);
         }
     }
+    return false;
 }
 
 // One Dense layer.  The bias goes into the GEMM only where the caller asks for it (bias_in_gemm: the Q/K/V
@@ -286,6 +293,7 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
 
     // (requests of at most 32 tokens are one pass over the weights whatever the arithmetic: they keep the fp32 kernels)
     const bool split = split_dense && M > 32;
+    bool operand_ready = false;
 
     T *prev_output = input_gpu;
     for (size_t l = 0; l < num_hidden_layers; ++l) {
@@ -294,27 +302,45 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
         T *out = layer_output[l & 1];
 
         if (split) {
-            dense_split(3 * H, M, H, w.qkv_split, layer_input, qkv_out, w.qkv_bias);
-            attention(batch_size, qkv_out, attention_mask);
-            dense_split(H, M, H, w.attention_output_split, context_out, attention_output, nullptr);
-            {
-                Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
-                cuBERT::layer_norm_(layer_input, attention_output, M, H, w.attention_output_bias, w.attention_norm_beta,
-                                    w.attention_norm_gamma, stream);
-            }
-            dense_split(I, M, H, w.intermediate_split, attention_output, intermediate_output, nullptr);
-            {
-                // bias + GELU straight into the two-term rows the output Dense reads
-                Timed t(profiler, Profiler::kBiasGelu, stream);
-                if constexpr (sizeof(T) == 4) {
+            if constexpr (sizeof(T) == 4) {
+                // split_operand holds the two-term rows of the next Dense input whenever the kernel before it could
+                // write them itself (LayerNorm, GELU); otherwise dense_split makes them from the fp32 rows
+                dense_split(3 * H, M, H, w.qkv_split, operand_ready ? nullptr : layer_input, qkv_out, w.qkv_bias);
+                const bool context_ready = attention(batch_size, qkv_out, attention_mask, split_operand);
+                dense_split(H, M, H, w.attention_output_split, context_ready ? nullptr : context_out, attention_output,
+                            nullptr);
+                {
+                    Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
+                    operand_ready = norm_writes_operand &&
+                                    cuBERT::layer_norm_split3(layer_input, attention_output, M, H, w.attention_output_bias,
+                                                              w.attention_norm_beta, w.attention_norm_gamma,
+                                                              split_operand, stream);
+                    if (!operand_ready) {
+                        norm_writes_operand = false;  // the hidden size is fixed per model: do not ask again
+                        cuBERT::layer_norm_(layer_input, attention_output, M, H, w.attention_output_bias,
+                                            w.attention_norm_beta, w.attention_norm_gamma, stream);
+                    }
+                }
+                dense_split(I, M, H, w.intermediate_split, operand_ready ? nullptr : attention_output,
+                            intermediate_output, nullptr);
+                {
+                    // bias + GELU straight into the two-term rows the output Dense reads
+                    Timed t(profiler, Profiler::kBiasGelu, stream);
                     cuBERT::bias_gelu_split3(intermediate_output, w.intermediate_bias, M, I, split_operand, stream);
                 }
-            }
-            dense_split(H, M, I, w.output_split, nullptr, out, nullptr);
-            {
-                Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
-                cuBERT::layer_norm_(attention_output, out, M, H, w.output_bias, w.output_norm_beta, w.output_norm_gamma,
-                                    stream);
+                dense_split(H, M, I, w.output_split, nullptr, out, nullptr);
+                {
+                    Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
+                    operand_ready = norm_writes_operand &&
+                                    cuBERT::layer_norm_split3(attention_output, out, M, H, w.output_bias,
+                                                              w.output_norm_beta, w.output_norm_gamma, split_operand,
+                                                              stream);
+                    if (!operand_ready) {
+                        norm_writes_operand = false;
+                        cuBERT::layer_norm_(attention_output, out, M, H, w.output_bias, w.output_norm_beta,
+                                            w.output_norm_gamma, stream);
+                    }
+                }
             }
             prev_output = out;
             continue;

@@ -80,7 +80,9 @@ private:
 
     void layout_weights();
     void layout_buffers();
-    void attention(size_t batch_size, const T *qkv, const int8_t *mask);
+    // context_out = attention(qkv); with `split_context` (fp32 models in the two-term Dense form) the one-launch
+    // kernel writes the context there as two-term rows instead and true is returned
+    bool attention(size_t batch_size, const T *qkv, const int8_t *mask, half *split_context = nullptr);
     // out[tokens, out_features] = in[tokens, in_features] * kernel (+ bias) (, GELU); returns whether bias and
     // activation were applied (false: the caller's fused kernel still has to).
     bool dense(int out_features, int tokens, int in_features, const T *kernel, const T *packed, const T *in, T *out,
@@ -96,6 +98,7 @@ private:
     bool keep_packed = false;          // Dense kernels are also kept in the few-token kernel's order
     bool transposed_kernels = false;   // Dense kernels are stored [out, in] instead of [in, out] (half precision)
     bool split_dense = false;          // fp32 model with Dense layers in the two-term fp16 form (opt-in)
+    bool norm_writes_operand = true;   // cleared when the LayerNorm that also writes two-term rows declines the hidden size
     bool fused_attention_fits = true;  // cleared when the one-launch attention kernel declines this model's shape
     size_t max_batch_size, seq_length, hidden_size, num_hidden_layers, num_attention_heads, intermediate_size;
 

@@ -58,6 +58,26 @@ struct Mma<float> {
 // Accumulator register i of lane (r = lane % 32, hh = lane / 32) is element (row, col) of the tile:
 __device__ __forceinline__ int acc_row(int i, int hh) { return (i >> 2) * 8 + hh * 4 + (i & 3); }
 
+// One element of the attention context.  split_width = 0: ctx[row, col] in the storage type.  split_width = W > 0
+// (fp32 only): `ctx` is really a buffer of halves with rows [hi | hi | lo] of W each, the two-term form the Dense
+// GEMM on the fp16 matrix cores reads (hi = fp16(v), lo = fp16(v - hi), clamped to the fp16 range).
+// (SPLIT is a compile-time choice so that the plain kernels are exactly what they were without it.)
+template <typename T, bool SPLIT>
+__device__ __forceinline__ void store_context(T *ctx, int ld_ctx, size_t row, int col, float v, int split_width) {
+    if constexpr (SPLIT) {
+        // v as the plain kernel would store it: rounded to fp32 before it is taken apart (without this the compiler
+        // fuses a product that made v into the subtraction below, and lo would belong to the unrounded value)
+        asm volatile("" : "+v"(v));
+        half_t *p = reinterpret_cast<half_t *>(ctx) + row * 3 * split_width + col;
+        const half_t hi = (half_t) fminf(fmaxf(v, -65504.f), 65504.f);
+        p[0] = hi;
+        p[split_width] = hi;
+        p[2 * split_width] = (half_t) fminf(fmaxf(v - (float) hi, -65504.f), 65504.f);
+    } else {
+        ctx[row * ld_ctx + col] = from_f32<T>(v);
+    }
+}
+
 // grid = (seq / 32 query tiles, key super-tiles, batch * heads); a wavefront computes 32 queries x (32 * NT) keys.
 template <typename T, int D, int NT>
 __global__ __launch_bounds__(kBlock) void attention_scores_kernel(const T *__restrict__ q, const T *__restrict__ k,
@@ -298,12 +318,12 @@ constexpr size_t fused_lds_bytes() {
 }
 
 // grid = batch * heads workgroups of KT wavefronts; seq = 32 * KT.
-template <typename T, int D, int KT>
+template <typename T, int D, int KT, bool SPLIT>
 __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__restrict__ q, const T *__restrict__ k,
                                                                      const T *__restrict__ v, int ld,
                                                                      const int8_t *__restrict__ mask,
                                                                      T *__restrict__ ctx, int ld_ctx, float alpha,
-                                                                     int heads) {
+                                                                     int heads, int split_width) {
     constexpr int V = Mma<T>::kVec;
     constexpr int kSteps = D / 2 / V;
     constexpr int kColTiles = D / 32;
@@ -435,11 +455,13 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
         }
     }
     // lane holds output column jt*32 + r and 16 query rows
-    T *dst = ctx + ((size_t) b * S + qt * 32) * ld_ctx + (size_t) h * D + r;
+    const size_t first_row = (size_t) b * S + qt * 32;
 #pragma unroll
     for (int jt = 0; jt < kColTiles; ++jt) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[(size_t) acc_row(i, hh) * ld_ctx + jt * 32] = from_f32<T>(out[jt][i]);
+        for (int i = 0; i < 16; ++i) {
+            store_context<T, SPLIT>(ctx, ld_ctx, first_row + acc_row(i, hh), h * D + jt * 32 + r, out[jt][i], split_width);
+        }
     }
 }
 
@@ -450,12 +472,12 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
 // used by one lane only), the four partial score tiles are added in wavefront order through LDS, every
 // wavefront repeats the (cheap) softmax, and P V is split into (column tile, key half), the two key halves
 // meeting in LDS again.  Same arithmetic and rounding as attention_fused_kernel, other summation order.
-template <typename T>
+template <typename T, bool SPLIT>
 __global__ __launch_bounds__(4 * kWave) void attention_small_kernel(const T *__restrict__ q, const T *__restrict__ k,
                                                                     const T *__restrict__ v, int ld,
                                                                     const int8_t *__restrict__ mask,
                                                                     T *__restrict__ ctx, int ld_ctx, float alpha,
-                                                                    int heads) {
+                                                                    int heads, int split_width) {
     constexpr int D = 64, S = 32;
     constexpr int V = Mma<T>::kVec;
     constexpr int kSteps = D / 8 / V;  // operand vectors per lane and contraction: a quarter of D over two lane halves
@@ -540,10 +562,10 @@ __global__ __launch_bounds__(4 * kWave) void attention_small_kernel(const T *__r
     }
     __syncthreads();
     if (kh == 0) {
-        T *dst = ctx + (row0) * ld_ctx + (size_t) h * D + jt * 32 + r;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            dst[(size_t) acc_row(i, hh) * ld_ctx] = from_f32<T>(out[i] + s_part[jt][i * kWave + lane]);
+            store_context<T, SPLIT>(ctx, ld_ctx, (size_t) row0 + acc_row(i, hh), h * D + jt * 32 + r,
+                             out[i] + s_part[jt][i * kWave + lane], split_width);
         }
     }
 }
@@ -563,12 +585,12 @@ __global__ __launch_bounds__(4 * kWave) void attention_small_kernel(const T *__r
 // all its tiles: there the shift cancels and the softmax runs over the raw scores, as in the reference).  Every
 // query row, padded or not, is still computed.  skip_masked_tiles = 0 (a mask that cannot be read as 32-bit
 // words) computes all tiles.
-template <typename T, int D>
+template <typename T, int D, bool SPLIT>
 __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restrict__ q, const T *__restrict__ k,
                                                                const T *__restrict__ v, int ld,
                                                                const int8_t *__restrict__ mask, T *__restrict__ ctx,
                                                                int ld_ctx, float alpha, int heads, int seq,
-                                                               int skip_masked_tiles) {
+                                                               int skip_masked_tiles, int split_width) {
     constexpr int V = Mma<T>::kVec;
     constexpr int kSteps = D / 2 / V;
     constexpr int kColTiles = D / 32;
@@ -755,7 +777,7 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
     if (hh == 0) factor[r] = 1.f / l;
     __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_wave_barrier();
-    T *dst = ctx + ((size_t) b * S + qt * 32) * ld_ctx + (size_t) h * D + r;
+    const size_t first_row = (size_t) b * S + qt * 32;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
         const Vec<float, 4> fr = load_vec<float, 4>(factor + g * 8 + hh * 4);
@@ -763,7 +785,8 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
         for (int jt = 0; jt < kColTiles; ++jt) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                dst[(size_t) acc_row(g * 4 + e, hh) * ld_ctx + jt * 32] = from_f32<T>(out[jt][g * 4 + e] * fr.v[e]);
+                store_context<T, SPLIT>(ctx, ld_ctx, first_row + acc_row(g * 4 + e, hh), h * D + jt * 32 + r,
+                                 out[jt][g * 4 + e] * fr.v[e], split_width);
             }
         }
     }
@@ -866,56 +889,85 @@ int attention_context(const T *probs, const T *v, int ld, T *ctx, int ld_ctx, in
 
 template <typename T, int D, int KT>
 int launch_fused_kt(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
-                    int batch, int heads, hipStream_t s) {
+                    int batch, int heads, int split_width, hipStream_t s) {
     constexpr size_t lds = fused_lds_bytes<T, D, KT>();
     if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
-    auto kernel = attention_fused_kernel<T, D, KT>;
+    if constexpr (sizeof(T) == 4) {
+        if (split_width > 0) {
+            auto kernel = attention_fused_kernel<T, D, KT, true>;
+            if (lds > 48 * 1024) {
+                static std::atomic<unsigned long long> raised{0};  // per instantiation
+                if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
+            }
+            return launch_untimed(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask,
+                                  ctx, ld_ctx, alpha, heads, split_width);
+        }
+    }
+    if (split_width > 0) return CUBERT_UNSUPPORTED;
+    auto kernel = attention_fused_kernel<T, D, KT, false>;
     if (lds > 48 * 1024) {
         static std::atomic<unsigned long long> raised{0};  // per instantiation
         if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
     }
     return launch_untimed(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask, ctx,
-                          ld_ctx, alpha, heads);
+                          ld_ctx, alpha, heads, split_width);
 }
 
 template <typename T, int D>
 int launch_fused(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
-                 int batch, int heads, int seq, hipStream_t s) {
+                 int batch, int heads, int seq, int split_width, hipStream_t s) {
     if constexpr (D == 64) {
         // fewer problems than compute units: split each over four wavefronts (5.3 -> 3.x us at 12 heads)
         if (seq == 32 && batch * heads <= 256 && (mask == nullptr || is_aligned(mask, 4))) {
-            return launch_untimed(attention_small_kernel<T>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q, k, v, ld,
-                                  mask, ctx, ld_ctx, alpha, heads);
+            if constexpr (sizeof(T) == 4) {
+                if (split_width > 0) {
+                    return launch_untimed(attention_small_kernel<T, true>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q,
+                                          k, v, ld, mask, ctx, ld_ctx, alpha, heads, split_width);
+                }
+            }
+            if (split_width > 0) return CUBERT_UNSUPPORTED;
+            return launch_untimed(attention_small_kernel<T, false>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q, k, v,
+                                  ld, mask, ctx, ld_ctx, alpha, heads, split_width);
         }
     }
     switch (seq / 32) {
-        case 1: return launch_fused_kt<T, D, 1>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, s);
-        case 2: return launch_fused_kt<T, D, 2>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, s);
-        case 3: return launch_fused_kt<T, D, 3>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, s);
-        case 4: return launch_fused_kt<T, D, 4>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, s);
+        case 1: return launch_fused_kt<T, D, 1>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width, s);
+        case 2: return launch_fused_kt<T, D, 2>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width, s);
+        case 3: return launch_fused_kt<T, D, 3>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width, s);
+        case 4: return launch_fused_kt<T, D, 4>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width, s);
         default: return CUBERT_UNSUPPORTED;
     }
 }
 
 template <typename T, int D>
 int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
-                 int batch, int heads, int seq, hipStream_t s) {
+                 int batch, int heads, int seq, int split_width, hipStream_t s) {
     constexpr int V = 16 / sizeof(T);
     if (seq > 512) return CUBERT_UNSUPPORTED;  // a workgroup has at most 16 wavefronts
     const size_t lds = (size_t) seq * (D + V) * sizeof(T) + (size_t) D * (seq + V) * sizeof(T) +
                        2 * (size_t) seq * sizeof(float);
     if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
-    auto kernel = attention_flash_kernel<T, D>;
+    const int skip_masked_tiles = mask != nullptr && is_aligned(mask, 4);  // seq is a multiple of 32
+    if constexpr (sizeof(T) == 4) {
+        if (split_width > 0) {
+            auto kernel = attention_flash_kernel<T, D, true>;
+            static std::atomic<unsigned long long> raised{0};  // per instantiation
+            if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
+            return launch_untimed(kernel, dim3(batch * heads), dim3(seq / 32 * kWave), (unsigned) lds, s, q, k, v, ld,
+                                  mask, ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles, split_width);
+        }
+    }
+    if (split_width > 0) return CUBERT_UNSUPPORTED;
+    auto kernel = attention_flash_kernel<T, D, false>;
     static std::atomic<unsigned long long> raised{0};  // per instantiation
     if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
-    const int skip_masked_tiles = mask != nullptr && is_aligned(mask, 4);  // seq is a multiple of 32
     return launch_untimed(kernel, dim3(batch * heads), dim3(seq / 32 * kWave), (unsigned) lds, s, q, k, v, ld, mask,
-                          ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles);
+                          ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles, split_width);
 }
 
 template <typename T>
 int attention_fused(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
-                    int batch, int heads, int seq, int head_size, void *stream) {
+                    int batch, int heads, int seq, int head_size, void *stream, int split_width = 0) {
     if (batch == 0 || heads == 0 || seq == 0) return 0;
     if (!q || !k || !v || !ctx || batch < 0 || heads < 0 || seq < 0 || head_size <= 0) return CUBERT_BAD_ARGUMENT;
     if (ld < heads * head_size) return CUBERT_BAD_ARGUMENT;
@@ -925,15 +977,15 @@ int attention_fused(const T *q, const T *k, const T *v, int ld, const int8_t *ma
     hipStream_t s = (hipStream_t) stream;
     if (seq > 128) {
         switch (head_size) {
-            case 32: return launch_flash<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, s);
-            case 64: return launch_flash<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, s);
+            case 32: return launch_flash<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, s);
+            case 64: return launch_flash<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, s);
             default: return CUBERT_UNSUPPORTED;  // head size 128 would spill the accumulators to scratch
         }
     }
     switch (head_size) {
-        case 32: return launch_fused<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, s);
-        case 64: return launch_fused<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, s);
-        default: return launch_fused<T, 128>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, s);
+        case 32: return launch_fused<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, s);
+        case 64: return launch_fused<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, s);
+        default: return launch_fused<T, 128>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, s);
     }
 }
 
@@ -968,6 +1020,15 @@ extern "C" int cubert_attention_fused_f32(const float *q, const float *k, const 
                                           int head_size, void *stream) {
     return cubert::attention_fused<float>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq_length, head_size,
                                           stream);
+}
+
+extern "C" int cubert_attention_fused_split3_f32(const float *q, const float *k, const float *v, int ld,
+                                                const int8_t *mask, cubert_half *split_ctx, float alpha, int batch,
+                                                int heads, int seq_length, int head_size, void *stream) {
+    if (split_ctx != nullptr && !cubert::is_aligned(split_ctx, 2)) return CUBERT_BAD_ARGUMENT;
+    const int hidden = heads * head_size;
+    return cubert::attention_fused<float>(q, k, v, ld, mask, reinterpret_cast<float *>(split_ctx), hidden, alpha, batch,
+                                          heads, seq_length, head_size, stream, hidden);
 }
 
 extern "C" int cubert_attention_fused_f16(const cubert_half *q, const cubert_half *k, const cubert_half *v, int ld,

@@ -44,11 +44,15 @@ __device__ __forceinline__ int uniform_i8(const int8_t *__restrict__ p, int inde
 
 // Normalise the row held in x[][] and store it.  gamma/beta were loaded before
 // the reduction so their latency overlaps it.
+// With `split_row` the stored values also go out as two-term fp16 rows [hi | hi | lo] (hi = fp16(y), lo = fp16(y - hi),
+// clamped to the fp16 range), the token operand of a Dense GEMM on the fp16 matrix cores (see split.hip).
 template <typename T, int VEC, int CHUNKS>
 __device__ __forceinline__ void ln_finish(float (&x)[CHUNKS][VEC], float sum, float sumsq, const Vec<T, VEC> (&g)[CHUNKS],
-                                          const Vec<T, VEC> (&b)[CHUNKS], T *__restrict__ out_row, int lane) {
+                                          const Vec<T, VEC> (&b)[CHUNKS], T *__restrict__ out_row, int lane,
+                                          half_t *__restrict__ split_row = nullptr) {
+    constexpr int H = kWave * VEC * CHUNKS;
     float mean, rstd;
-    ln_stats(sum, sumsq, kWave * VEC * CHUNKS, mean, rstd);
+    ln_stats(sum, sumsq, H, mean, rstd);
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         Vec<T, VEC> o;
@@ -57,13 +61,27 @@ __device__ __forceinline__ void ln_finish(float (&x)[CHUNKS][VEC], float sum, fl
             o.v[i] = from_f32<T>(to_f32(b[c].v[i]) + (to_f32(g[c].v[i]) * rstd) * (x[c][i] - mean));
         }
         store_vec<T, VEC>(out_row + (c * kWave + lane) * VEC, o);
+        if (split_row != nullptr) {  // (uniform)
+            Vec<half_t, VEC> hi, lo;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                const float y = to_f32(o.v[i]);
+                hi.v[i] = (half_t) fminf(fmaxf(y, -65504.f), 65504.f);
+                lo.v[i] = (half_t) fminf(fmaxf(y - (float) hi.v[i], -65504.f), 65504.f);
+            }
+            half_t *at = split_row + (c * kWave + lane) * VEC;
+            store_vec<half_t, VEC>(at, hi);
+            store_vec<half_t, VEC>(at + H, hi);
+            store_vec<half_t, VEC>(at + 2 * H, lo);
+        }
     }
 }
 
-template <typename T, int VEC, int CHUNKS, bool HAS_BIAS>
+template <typename T, int VEC, int CHUNKS, bool HAS_BIAS, bool SPLIT = false>
 __global__ __launch_bounds__(kBlock) void bias_res_ln_kernel(T *__restrict__ inout, const T *__restrict__ residual,
                                                              const T *__restrict__ bias, const T *__restrict__ beta,
-                                                             const T *__restrict__ gamma, int rows) {
+                                                             const T *__restrict__ gamma, int rows,
+                                                             half_t *__restrict__ split_out) {
     constexpr int H = kWave * VEC * CHUNKS;
     const int row = blockIdx.x * kRowsPerBlock + wave_in_block();
     if (row >= rows) return;
@@ -101,7 +119,7 @@ __global__ __launch_bounds__(kBlock) void bias_res_ln_kernel(T *__restrict__ ino
             sumsq += v * v;
         }
     }
-    ln_finish<T, VEC, CHUNKS>(x, sum, sumsq, g, be, io, lane);
+    ln_finish<T, VEC, CHUNKS>(x, sum, sumsq, g, be, io, lane, SPLIT ? split_out + (size_t) row * 3 * H : nullptr);
 }
 
 template <typename T, int VEC, int CHUNKS>
@@ -332,9 +350,9 @@ int bias_res_ln(T *inout, const T *residual, const T *bias, const T *beta, const
     if (hidden == kWave * VEC * CHUNKS && vector_ok<T>(hidden, VEC, {inout, residual, bias, beta, gamma})) { \
         if (bias != nullptr)                                                                             \
             return launch(bias_res_ln_kernel<T, VEC, CHUNKS, true>, grid, block, s, inout, residual, bias, beta, gamma, \
-                          rows);                                                                         \
+                          rows, nullptr);                                                                \
         return launch(bias_res_ln_kernel<T, VEC, CHUNKS, false>, grid, block, s, inout, residual, bias, beta, gamma, \
-                      rows);                                                                             \
+                      rows, nullptr);                                                                    \
     }
     CUBERT_LN_CASE(V, 1)
     CUBERT_LN_CASE(V, 2)
@@ -350,6 +368,34 @@ int bias_res_ln(T *inout, const T *residual, const T *bias, const T *beta, const
 #undef CUBERT_LN_CASE
     return launch(ln_generic_kernel<T, false>, grid, block, s, inout, residual, bias, nullptr, nullptr, nullptr, nullptr,
                   nullptr, beta, gamma, rows, hidden, 1);
+}
+
+// bias + residual + LayerNorm of fp32 rows, in place, and the result again as two-term fp16 rows in split_out
+// [rows, 3 * hidden]; only the register-resident shapes (hidden = 256 k), anything else is declined.
+int bias_res_ln_split3(float *inout, const float *residual, const float *bias, const float *beta, const float *gamma,
+                       int rows, int hidden, half_t *split_out, void *stream) {
+    if (rows < 0 || hidden <= 0 || !inout || !residual || !beta || !gamma || !split_out) return CUBERT_BAD_ARGUMENT;
+    if (rows == 0) return 0;
+    hipStream_t s = (hipStream_t) stream;
+    dim3 grid((rows + kRowsPerBlock - 1) / kRowsPerBlock), block(kBlock);
+    if (!is_aligned(split_out, 8)) return CUBERT_UNSUPPORTED;
+#define CUBERT_LN_SPLIT_CASE(CHUNKS)                                                                                  \
+    if (hidden == kWave * 4 * CHUNKS && vector_ok<float>(hidden, 4, {inout, residual, bias, beta, gamma})) {         \
+        if (bias != nullptr)                                                                                          \
+            return launch(bias_res_ln_kernel<float, 4, CHUNKS, true, true>, grid, block, s, inout, residual, bias, beta, \
+                          gamma, rows, split_out);                                                                    \
+        return launch(bias_res_ln_kernel<float, 4, CHUNKS, false, true>, grid, block, s, inout, residual, bias, beta,  \
+                      gamma, rows, split_out);                                                                        \
+    }
+    CUBERT_LN_SPLIT_CASE(1)
+    CUBERT_LN_SPLIT_CASE(2)
+    CUBERT_LN_SPLIT_CASE(3)
+    CUBERT_LN_SPLIT_CASE(4)
+    CUBERT_LN_SPLIT_CASE(5)
+    CUBERT_LN_SPLIT_CASE(6)
+    CUBERT_LN_SPLIT_CASE(8)
+#undef CUBERT_LN_SPLIT_CASE
+    return CUBERT_UNSUPPORTED;
 }
 
 template <typename T>
@@ -399,6 +445,13 @@ using cubert::half_t;
 extern "C" int cubert_bias_res_ln_f32(float *inout, const float *residual, const float *bias, const float *beta,
                                       const float *gamma, int rows, int hidden, void *stream) {
     return cubert::bias_res_ln<float>(inout, residual, bias, beta, gamma, rows, hidden, stream);
+}
+
+extern "C" int cubert_bias_res_ln_split3_f32(float *inout, const float *residual, const float *bias, const float *beta,
+                                             const float *gamma, int rows, int hidden, cubert_half *split_out,
+                                             void *stream) {
+    return cubert::bias_res_ln_split3(inout, residual, bias, beta, gamma, rows, hidden, (cubert::half_t *) split_out,
+                                      stream);
 }
 
 extern "C" int cubert_bias_res_ln_f16(cubert_half *inout, const cubert_half *residual, const cubert_half *bias,

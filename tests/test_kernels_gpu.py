@@ -409,6 +409,50 @@ def test_bias_gelu_split3_against_oracle(K, rows, width):
     assert np.all(np.abs(value - inplace) <= np.maximum(np.abs(inplace) * 2.0 ** -21, 2.0 ** -24))
 
 
+@pytest.mark.parametrize("rows,hidden,with_bias", [(37, 768, True), (5, 1024, False), (4, 256, True), (3, 2048, True)])
+def test_bias_res_ln_split3_equals_ln_then_split(K, rows, hidden, with_bias):
+    rng = np.random.default_rng(hidden + rows)
+    x = rng.normal(0, 1, (rows, hidden)).astype(np.float32)
+    res = rng.normal(0, 1, (rows, hidden)).astype(np.float32)
+    bias = rng.normal(0, 0.1, hidden).astype(np.float32) if with_bias else None
+    beta = rng.normal(0, 0.1, hidden).astype(np.float32)
+    gamma = rng.normal(1, 0.1, hidden).astype(np.float32)
+    args = [dev(res), None if bias is None else dev(bias), dev(beta), dev(gamma)]
+    plain = K.bias_res_ln_(dev(x), *args)
+    want_split = K.split3(plain)
+    inout = dev(x)
+    got_split = K.bias_res_ln_split3_(inout, *args)
+    assert got_split is not None
+    torch.cuda.synchronize()
+    assert torch.equal(inout, plain)             # the fp32 result is the plain kernel's, bit for bit
+    assert torch.equal(got_split, want_split)    # and its two-term rows are those of the split kernel
+    assert_close(host(inout), oracle.layer_norm_(res, x + (0 if bias is None else bias), beta, gamma), FP32_TOL, "LN")
+
+
+@pytest.mark.parametrize("batch,heads,seq,d", [(1, 12, 32, 64), (24, 12, 32, 64), (3, 4, 128, 64), (2, 3, 64, 32),
+                                               (1, 2, 256, 64), (2, 2, 96, 128)])
+def test_attention_fused_split3_equals_attention_then_split(K, batch, heads, seq, d):
+    rng = np.random.default_rng(batch + heads + seq + d)
+    H = heads * d
+    qkv = dev(rng.normal(0, 1, (batch * seq, 3 * H)).astype(np.float32))
+    mask = (rng.random((batch, seq)) < 0.7).astype(np.int8)
+    mask[:, 0] = 1
+    mask = dev(mask)
+    alpha = 1.0 / math.sqrt(d)
+    plain = K.attention_fused(qkv, mask, batch, heads, seq, d, alpha)
+    assert plain is not None
+    got = K.attention_fused_split3(qkv, mask, batch, heads, seq, d, alpha)
+    assert got is not None
+    torch.cuda.synchronize()
+    assert torch.equal(got, K.split3(plain))  # the same context values, written in the other form
+
+
+def test_bias_res_ln_split3_declines_other_hidden_sizes(K):
+    x = dev(np.zeros((2, 100), np.float32))
+    v = dev(np.ones(100, np.float32))
+    assert K.bias_res_ln_split3_(x, x.clone(), None, v, v) is None
+
+
 @pytest.mark.parametrize("tokens,in_features,out_features", [(4096, 768, 2304), (200, 3072, 768), (64, 128, 512),
                                                              (33, 40, 24)])
 def test_two_term_dense_matches_fp32_dense(K, tokens, in_features, out_features):

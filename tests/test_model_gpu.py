@@ -213,7 +213,9 @@ def test_two_term_fp16_dense_of_an_fp32_model(cb, monkeypatch):
     bert.profile(["dense_split", "dense_gemm"])
     got = bert.forward(ids, mask, seg)
     counts = bert.profile_read()
-    assert counts["dense_split"][1] == 3 * m["layers"], counts   # the form was in use
+    # the form was in use: one split pass, for the first layer's input (the other Dense inputs are written in two-term
+    # form by the attention, LayerNorm and GELU kernels themselves)
+    assert counts["dense_split"][1] == 1 and counts["dense_gemm"][1] >= 4 * m["layers"], counts
     one = bert.forward(ids[:1], mask[:1], seg[:1])               # 32 tokens: fp32 few-token kernels
     assert "dense_split" not in bert.profile_read()
     bert.close()
