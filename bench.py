@@ -169,7 +169,14 @@ def main():
                     help="skip the extra leg that repeats the steps with CUBERT_FP32_DENSE=f16x3 (fp32 workloads)")
     ap.add_argument("--device-only", action="store_true",
                     help="only the device-resident steps (no host-path / batch-1 latency loops): for profiler runs")
+    ap.add_argument("--fp32-dense", choices=["f32", "f16x3"], default=None,
+                    help="f16x3: open the model with CUBERT_FP32_DENSE=f16x3 (the opt-in two-term fp16 Dense form of fp32 "
+                         "models); default: whatever the environment says, normally the fp32 GEMM")
     args = ap.parse_args()
+    if args.fp32_dense == "f16x3":
+        os.environ["CUBERT_FP32_DENSE"] = "f16x3"
+    elif args.fp32_dense == "f32":
+        os.environ.pop("CUBERT_FP32_DENSE", None)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (replicas on several GPUs share nothing); "
               "run with --gpus 1", file=sys.stderr)
