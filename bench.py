@@ -53,7 +53,7 @@ MEASURED_TRAFFIC = {
 
 
 def two_term_dense():
-    """CUBERT_FP32_DENSE=f16x3 in the environment: fp32 models run their Dense layers of more than 32 tokens on the
+    """CUBERT_FP32_DENSE=f16x3 in the environment: fp32 models run their Dense layers (requests of at least 384 tokens) on the
     fp16 matrix cores from two-term operands (opt-in; the default is the fp32 GEMM)."""
     return os.environ.get("CUBERT_FP32_DENSE") == "f16x3"
 
@@ -65,7 +65,7 @@ def algorithmic_bytes(cfg):
     H, I, A = m["hidden"], m["intermediate"], m["heads"]
     e = 4 if cfg["dtype"] == "f32" else 2
     M = B * S
-    if two_term_dense() and e == 4 and M > 32:
+    if two_term_dense() and e == 4 and M >= 384:
         # bias+GELU reads fp32 and writes [hi | hi | lo] fp16 rows; the LayerNorm writes both forms
         extra = {"bias_gelu": M * I * (4 + 6) + I * 4, "bias_res_ln": 3 * M * H * 4 + 3 * H * 4 + 6 * M * H,
                  "dense_split": M * H * (4 + 6)}
@@ -285,7 +285,7 @@ def main():
 
     # ---- the same steps with the opt-in two-term fp16 Dense form of fp32 models (reported beside `value`, never as it)
     two_term = None
-    if not half and B * S > 32 and not two_term_dense() and not args.device_only and not args.no_two_term:
+    if not half and B * S >= 384 and not two_term_dense() and not args.device_only and not args.no_two_term:
         os.environ["CUBERT_FP32_DENSE"] = "f16x3"  # read when a model is opened
         try:
             other = cubert_amd.Bert(w, B, S, m["layers"], m["heads"], 0)

@@ -46,7 +46,7 @@ Transformer<T>::Transformer(void *cublas, const std::string &var_prefix,
     transposed_kernels = sizeof(T) == 2;
     const char *dense_mode = std::getenv("CUBERT_FP32_DENSE");
     split_dense = sizeof(T) == 4 && dense_mode != nullptr && std::string(dense_mode) == "f16x3" &&
-                  max_batch_size * seq_length > 32;
+                  max_batch_size * seq_length >= kTwoTermMinTokens;
 
     // Weight names as the reference resolves them (Transformer.cpp:54-101, AttentionSelf.cpp:27-44);
     // a missing name throws std::out_of_range from unordered_map::at, as it does there.
@@ -291,8 +291,9 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
     void *stream = cuBERT::blas_get_stream(cublas);
     const int M = (int) (batch_size * seq_length), H = (int) hidden_size, I = (int) intermediate_size;
 
-    // (requests of at most 32 tokens are one pass over the weights whatever the arithmetic: they keep the fp32 kernels)
-    const bool split = split_dense && M > 32;
+    // (small requests are bound by the pass over the weights, which are 6 bytes per parameter in two-term form and 4
+    // in fp32: they keep the fp32 kernels)
+    const bool split = split_dense && (size_t) M >= kTwoTermMinTokens;
     bool operand_ready = false;
 
     T *prev_output = input_gpu;

@@ -16,8 +16,9 @@
 // buffers per layer); weights live in one device allocation.  A half-precision model whose seq_length allows
 // requests of at most 32 tokens also keeps its four Dense kernels in the few-token GEMM kernel's own order.
 //
-// CUBERT_FP32_DENSE=f16x3 in the environment when an fp32 model is opened makes its Dense layers of more than 32
-// tokens run on the fp16 matrix cores: every fp32 operand is written as the sum of two fp16 numbers and the
+// CUBERT_FP32_DENSE=f16x3 in the environment when an fp32 model is opened makes its Dense layers run on the fp16
+// matrix cores for requests of at least 384 tokens (measured break-even at BERT-base: below it the GEMMs are bound
+// by reading the weights, and two-term weights are the larger ones): every fp32 operand is written as the sum of two fp16 numbers and the
 // product as hi*hi + hi*lo + lo*hi with fp32 accumulation (one GEMM over three times the reduction length), which
 // keeps the error of an fp32 GEMM for activations inside the fp16 range (|x| <= 65504; see kernels/split.hip).
 // Everything between the GEMMs stays fp32.  The default is the fp32 GEMM.
@@ -59,6 +60,7 @@ public:
 
 private:
     // A Dense kernel for the two-term fp16 form: rows [hi | lo | hi] of scale * W^T, [out, 3 * in]; unscale = 1 / scale
+    static constexpr size_t kTwoTermMinTokens = 384;
     struct SplitKernel {
         half *weights = nullptr;
         float unscale = 1.f;
