@@ -202,7 +202,8 @@ bool Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *ma
         Timed t(profiler, Profiler::kAttentionFused, stream);
         if constexpr (sizeof(T) == 4) {
             if (split_context != nullptr &&
-                cuBERT::attention_fused_split3(Q, K, V, ld, mask, split_context, alpha, B, A, S, d, stream)) {
+                cuBERT::attention_fused_split3(Q, K, V, ld, mask, kTwoTermActivationScale, split_context, alpha, B, A, S,
+                                               d, stream)) {
                 return true;
             }
         }
@@ -274,10 +275,11 @@ void Transformer<T>::dense_split(int out_features, int tokens, int in_features, 
         void *stream = cuBERT::blas_get_stream(cublas);
         if (in != nullptr) {
             Timed t(profiler, Profiler::kDenseSplit, stream);
-            cuBERT::split3(in, tokens, in_features, 1.f, false, split_operand, stream);
+            cuBERT::split3(in, tokens, in_features, kTwoTermActivationScale, false, split_operand, stream);
         }
         Timed t(profiler, Profiler::kDenseGemm, stream);
-        cuBERT::blas_gemm_f16_f32(cublas, true, false, out_features, tokens, 3 * in_features, kernel.unscale,
+        cuBERT::blas_gemm_f16_f32(cublas, true, false, out_features, tokens, 3 * in_features,
+                                  kernel.unscale / kTwoTermActivationScale,
                                   kernel.weights, 3 * in_features, split_operand, 3 * in_features, 0.f, out,
                                   out_features, bias);
     } else {
@@ -315,7 +317,7 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
                     operand_ready = norm_writes_operand &&
                                     cuBERT::layer_norm_split3(layer_input, attention_output, M, H, w.attention_output_bias,
                                                               w.attention_norm_beta, w.attention_norm_gamma,
-                                                              split_operand, stream);
+                                                              kTwoTermActivationScale, split_operand, stream);
                     if (!operand_ready) {
                         norm_writes_operand = false;  // the hidden size is fixed per model: do not ask again
                         cuBERT::layer_norm_(layer_input, attention_output, M, H, w.attention_output_bias,
@@ -327,15 +329,16 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
                 {
                     // bias + GELU straight into the two-term rows the output Dense reads
                     Timed t(profiler, Profiler::kBiasGelu, stream);
-                    cuBERT::bias_gelu_split3(intermediate_output, w.intermediate_bias, M, I, split_operand, stream);
+                    cuBERT::bias_gelu_split3(intermediate_output, w.intermediate_bias, M, I, kTwoTermActivationScale,
+                                             split_operand, stream);
                 }
                 dense_split(H, M, I, w.output_split, nullptr, out, nullptr);
                 {
                     Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
                     operand_ready = norm_writes_operand &&
                                     cuBERT::layer_norm_split3(attention_output, out, M, H, w.output_bias,
-                                                              w.output_norm_beta, w.output_norm_gamma, split_operand,
-                                                              stream);
+                                                              w.output_norm_beta, w.output_norm_gamma,
+                                                              kTwoTermActivationScale, split_operand, stream);
                     if (!operand_ready) {
                         norm_writes_operand = false;
                         cuBERT::layer_norm_(attention_output, out, M, H, w.output_bias, w.output_norm_beta,

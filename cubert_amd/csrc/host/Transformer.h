@@ -20,7 +20,7 @@
 // matrix cores for requests of at least 384 tokens (measured break-even at BERT-base: below it the GEMMs are bound
 // by reading the weights, and two-term weights are the larger ones): every fp32 operand is written as the sum of two fp16 numbers and the
 // product as hi*hi + hi*lo + lo*hi with fp32 accumulation (one GEMM over three times the reduction length), which
-// keeps the error of an fp32 GEMM for activations inside the fp16 range (|x| <= 65504; see kernels/split.hip).
+// keeps the error of an fp32 GEMM for activations up to 2^12 in size (see kernels/split.hip).
 // Everything between the GEMMs stays fp32.  The default is the fp32 GEMM.
 #ifndef CUBERT_HOST_TRANSFORMER_H
 #define CUBERT_HOST_TRANSFORMER_H
@@ -61,6 +61,9 @@ public:
 private:
     // A Dense kernel for the two-term fp16 form: rows [hi | lo | hi] of scale * W^T, [out, 3 * in]; unscale = 1 / scale
     static constexpr size_t kTwoTermMinTokens = 384;
+    // activations are multiplied by this before they are taken apart (undone by the GEMM's alpha): rows whose
+    // entries are of order 2^-7 .. 2^12 keep full accuracy (fp16 subnormals below, clamping above)
+    static constexpr float kTwoTermActivationScale = 16.f;
     struct SplitKernel {
         half *weights = nullptr;
         float unscale = 1.f;

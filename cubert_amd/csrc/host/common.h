@@ -120,24 +120,26 @@ inline void split3(const float *in, int rows, int width, float scale, bool lo_in
 }
 // false: the shape is not one the fused kernel takes (the caller runs layer_norm_ and split3)
 inline bool layer_norm_split3(const float *in, float *inout, int rows, int channels, const float *bias,
-                              const float *beta, const float *gamma, half *split_out, void *stream) {
-    const int rc = cubert_bias_res_ln_split3_f32(inout, in, bias, beta, gamma, rows, channels, h(split_out), stream);
+                              const float *beta, const float *gamma, float scale, half *split_out, void *stream) {
+    const int rc = cubert_bias_res_ln_split3_f32(inout, in, bias, beta, gamma, rows, channels, scale, h(split_out),
+                                                 stream);
     if (rc == CUBERT_UNSUPPORTED) return false;
     CUBERT_CHECK(rc);
     return true;
 }
 // the one-launch attention core with its context in two-term rows; false when the shape is not taken
 inline bool attention_fused_split3(const float *q, const float *k, const float *v, int ld, const int8_t *mask,
-                                   half *split_ctx, float alpha, int batch, int heads, int seq, int head_size,
-                                   void *stream) {
-    const int rc = cubert_attention_fused_split3_f32(q, k, v, ld, mask, h(split_ctx), alpha, batch, heads, seq, head_size,
-                                                     stream);
+                                   float scale, half *split_ctx, float alpha, int batch, int heads, int seq,
+                                   int head_size, void *stream) {
+    const int rc = cubert_attention_fused_split3_f32(q, k, v, ld, mask, scale, h(split_ctx), alpha, batch, heads, seq,
+                                                     head_size, stream);
     if (rc == CUBERT_UNSUPPORTED) return false;
     CUBERT_CHECK(rc);
     return true;
 }
-inline void bias_gelu_split3(const float *in, const float *bias, int rows, int width, half *out, void *stream) {
-    CUBERT_CHECK(cubert_bias_gelu_split3_f32(in, bias, rows, width, h(out), stream));
+inline void bias_gelu_split3(const float *in, const float *bias, int rows, int width, float scale, half *out,
+                             void *stream) {
+    CUBERT_CHECK(cubert_bias_gelu_split3_f32(in, bias, rows, width, scale, h(out), stream));
 }
 
 inline void transpose(const float *in, int rows, int cols, float *out, void *stream) {

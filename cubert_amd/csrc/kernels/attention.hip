@@ -59,15 +59,18 @@ struct Mma<float> {
 __device__ __forceinline__ int acc_row(int i, int hh) { return (i >> 2) * 8 + hh * 4 + (i & 3); }
 
 // One element of the attention context.  split_width = 0: ctx[row, col] in the storage type.  split_width = W > 0
-// (fp32 only): `ctx` is really a buffer of halves with rows [hi | hi | lo] of W each, the two-term form the Dense
-// GEMM on the fp16 matrix cores reads (hi = fp16(v), lo = fp16(v - hi), clamped to the fp16 range).
+// (fp32 only): `ctx` is really a buffer of halves with rows [hi | hi | lo] of W each, the two-term form of
+// split_scale * v that the Dense GEMM on the fp16 matrix cores reads (hi = fp16(.), lo = fp16(. - hi), clamped to
+// the fp16 range).
 // (SPLIT is a compile-time choice so that the plain kernels are exactly what they were without it.)
 template <typename T, bool SPLIT>
-__device__ __forceinline__ void store_context(T *ctx, int ld_ctx, size_t row, int col, float v, int split_width) {
+__device__ __forceinline__ void store_context(T *ctx, int ld_ctx, size_t row, int col, float v, int split_width,
+                                              float split_scale) {
     if constexpr (SPLIT) {
         // v as the plain kernel would store it: rounded to fp32 before it is taken apart (without this the compiler
         // fuses a product that made v into the subtraction below, and lo would belong to the unrounded value)
         asm volatile("" : "+v"(v));
+        v *= split_scale;
         half_t *p = reinterpret_cast<half_t *>(ctx) + row * 3 * split_width + col;
         const half_t hi = (half_t) fminf(fmaxf(v, -65504.f), 65504.f);
         p[0] = hi;
@@ -323,7 +326,7 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
                                                                      const T *__restrict__ v, int ld,
                                                                      const int8_t *__restrict__ mask,
                                                                      T *__restrict__ ctx, int ld_ctx, float alpha,
-                                                                     int heads, int split_width) {
+                                                                     int heads, int split_width, float split_scale) {
     constexpr int V = Mma<T>::kVec;
     constexpr int kSteps = D / 2 / V;
     constexpr int kColTiles = D / 32;
@@ -460,7 +463,8 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
     for (int jt = 0; jt < kColTiles; ++jt) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            store_context<T, SPLIT>(ctx, ld_ctx, first_row + acc_row(i, hh), h * D + jt * 32 + r, out[jt][i], split_width);
+            store_context<T, SPLIT>(ctx, ld_ctx, first_row + acc_row(i, hh), h * D + jt * 32 + r, out[jt][i], split_width,
+                                    split_scale);
         }
     }
 }
@@ -477,7 +481,7 @@ __global__ __launch_bounds__(4 * kWave) void attention_small_kernel(const T *__r
                                                                     const T *__restrict__ v, int ld,
                                                                     const int8_t *__restrict__ mask,
                                                                     T *__restrict__ ctx, int ld_ctx, float alpha,
-                                                                    int heads, int split_width) {
+                                                                    int heads, int split_width, float split_scale) {
     constexpr int D = 64, S = 32;
     constexpr int V = Mma<T>::kVec;
     constexpr int kSteps = D / 8 / V;  // operand vectors per lane and contraction: a quarter of D over two lane halves
@@ -565,7 +569,7 @@ __global__ __launch_bounds__(4 * kWave) void attention_small_kernel(const T *__r
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             store_context<T, SPLIT>(ctx, ld_ctx, (size_t) row0 + acc_row(i, hh), h * D + jt * 32 + r,
-                             out[i] + s_part[jt][i * kWave + lane], split_width);
+                             out[i] + s_part[jt][i * kWave + lane], split_width, split_scale);
         }
     }
 }
@@ -590,7 +594,8 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
                                                                const T *__restrict__ v, int ld,
                                                                const int8_t *__restrict__ mask, T *__restrict__ ctx,
                                                                int ld_ctx, float alpha, int heads, int seq,
-                                                               int skip_masked_tiles, int split_width) {
+                                                               int skip_masked_tiles, int split_width,
+                                                               float split_scale) {
     constexpr int V = Mma<T>::kVec;
     constexpr int kSteps = D / 2 / V;
     constexpr int kColTiles = D / 32;
@@ -786,7 +791,7 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 store_context<T, SPLIT>(ctx, ld_ctx, first_row + acc_row(g * 4 + e, hh), h * D + jt * 32 + r,
-                                 out[jt][g * 4 + e] * fr.v[e], split_width);
+                                 out[jt][g * 4 + e] * fr.v[e], split_width, split_scale);
             }
         }
     }
@@ -889,7 +894,7 @@ int attention_context(const T *probs, const T *v, int ld, T *ctx, int ld_ctx, in
 
 template <typename T, int D, int KT>
 int launch_fused_kt(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
-                    int batch, int heads, int split_width, hipStream_t s) {
+                    int batch, int heads, int split_width, float split_scale, hipStream_t s) {
     constexpr size_t lds = fused_lds_bytes<T, D, KT>();
     if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
     if constexpr (sizeof(T) == 4) {
@@ -900,7 +905,7 @@ int launch_fused_kt(const T *q, const T *k, const T *v, int ld, const int8_t *ma
                 if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
             }
             return launch_untimed(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask,
-                                  ctx, ld_ctx, alpha, heads, split_width);
+                                  ctx, ld_ctx, alpha, heads, split_width, split_scale);
         }
     }
     if (split_width > 0) return CUBERT_UNSUPPORTED;
@@ -910,38 +915,46 @@ int launch_fused_kt(const T *q, const T *k, const T *v, int ld, const int8_t *ma
         if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
     }
     return launch_untimed(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask, ctx,
-                          ld_ctx, alpha, heads, split_width);
+                          ld_ctx, alpha, heads, split_width, split_scale);
 }
 
 template <typename T, int D>
 int launch_fused(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
-                 int batch, int heads, int seq, int split_width, hipStream_t s) {
+                 int batch, int heads, int seq, int split_width, float split_scale, hipStream_t s) {
     if constexpr (D == 64) {
         // fewer problems than compute units: split each over four wavefronts (5.3 -> 3.x us at 12 heads)
         if (seq == 32 && batch * heads <= 256 && (mask == nullptr || is_aligned(mask, 4))) {
             if constexpr (sizeof(T) == 4) {
                 if (split_width > 0) {
                     return launch_untimed(attention_small_kernel<T, true>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q,
-                                          k, v, ld, mask, ctx, ld_ctx, alpha, heads, split_width);
+                                          k, v, ld, mask, ctx, ld_ctx, alpha, heads, split_width, split_scale);
                 }
             }
             if (split_width > 0) return CUBERT_UNSUPPORTED;
             return launch_untimed(attention_small_kernel<T, false>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q, k, v,
-                                  ld, mask, ctx, ld_ctx, alpha, heads, split_width);
+                                  ld, mask, ctx, ld_ctx, alpha, heads, split_width, split_scale);
         }
     }
     switch (seq / 32) {
-        case 1: return launch_fused_kt<T, D, 1>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width, s);
-        case 2: return launch_fused_kt<T, D, 2>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width, s);
-        case 3: return launch_fused_kt<T, D, 3>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width, s);
-        case 4: return launch_fused_kt<T, D, 4>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width, s);
+        case 1:
+            return launch_fused_kt<T, D, 1>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width,
+                                             split_scale, s);
+        case 2:
+            return launch_fused_kt<T, D, 2>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width,
+                                             split_scale, s);
+        case 3:
+            return launch_fused_kt<T, D, 3>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width,
+                                             split_scale, s);
+        case 4:
+            return launch_fused_kt<T, D, 4>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width,
+                                             split_scale, s);
         default: return CUBERT_UNSUPPORTED;
     }
 }
 
 template <typename T, int D>
 int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
-                 int batch, int heads, int seq, int split_width, hipStream_t s) {
+                 int batch, int heads, int seq, int split_width, float split_scale, hipStream_t s) {
     constexpr int V = 16 / sizeof(T);
     if (seq > 512) return CUBERT_UNSUPPORTED;  // a workgroup has at most 16 wavefronts
     const size_t lds = (size_t) seq * (D + V) * sizeof(T) + (size_t) D * (seq + V) * sizeof(T) +
@@ -954,7 +967,7 @@ int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask,
             static std::atomic<unsigned long long> raised{0};  // per instantiation
             if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
             return launch_untimed(kernel, dim3(batch * heads), dim3(seq / 32 * kWave), (unsigned) lds, s, q, k, v, ld,
-                                  mask, ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles, split_width);
+                                  mask, ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles, split_width, split_scale);
         }
     }
     if (split_width > 0) return CUBERT_UNSUPPORTED;
@@ -962,12 +975,13 @@ int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask,
     static std::atomic<unsigned long long> raised{0};  // per instantiation
     if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
     return launch_untimed(kernel, dim3(batch * heads), dim3(seq / 32 * kWave), (unsigned) lds, s, q, k, v, ld, mask,
-                          ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles, split_width);
+                          ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles, split_width, split_scale);
 }
 
 template <typename T>
 int attention_fused(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
-                    int batch, int heads, int seq, int head_size, void *stream, int split_width = 0) {
+                    int batch, int heads, int seq, int head_size, void *stream, int split_width = 0,
+                    float split_scale = 1.f) {
     if (batch == 0 || heads == 0 || seq == 0) return 0;
     if (!q || !k || !v || !ctx || batch < 0 || heads < 0 || seq < 0 || head_size <= 0) return CUBERT_BAD_ARGUMENT;
     if (ld < heads * head_size) return CUBERT_BAD_ARGUMENT;
@@ -977,15 +991,25 @@ int attention_fused(const T *q, const T *k, const T *v, int ld, const int8_t *ma
     hipStream_t s = (hipStream_t) stream;
     if (seq > 128) {
         switch (head_size) {
-            case 32: return launch_flash<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, s);
-            case 64: return launch_flash<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, s);
+            case 32:
+                return launch_flash<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width,
+                                           split_scale, s);
+            case 64:
+                return launch_flash<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width,
+                                           split_scale, s);
             default: return CUBERT_UNSUPPORTED;  // head size 128 would spill the accumulators to scratch
         }
     }
     switch (head_size) {
-        case 32: return launch_fused<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, s);
-        case 64: return launch_fused<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, s);
-        default: return launch_fused<T, 128>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, s);
+        case 32:
+            return launch_fused<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, split_scale,
+                                       s);
+        case 64:
+            return launch_fused<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, split_scale,
+                                       s);
+        default:
+            return launch_fused<T, 128>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, split_scale,
+                                        s);
     }
 }
 
@@ -1023,12 +1047,12 @@ extern "C" int cubert_attention_fused_f32(const float *q, const float *k, const 
 }
 
 extern "C" int cubert_attention_fused_split3_f32(const float *q, const float *k, const float *v, int ld,
-                                                const int8_t *mask, cubert_half *split_ctx, float alpha, int batch,
-                                                int heads, int seq_length, int head_size, void *stream) {
+                                                const int8_t *mask, float scale, cubert_half *split_ctx, float alpha,
+                                                int batch, int heads, int seq_length, int head_size, void *stream) {
     if (split_ctx != nullptr && !cubert::is_aligned(split_ctx, 2)) return CUBERT_BAD_ARGUMENT;
     const int hidden = heads * head_size;
     return cubert::attention_fused<float>(q, k, v, ld, mask, reinterpret_cast<float *>(split_ctx), hidden, alpha, batch,
-                                          heads, seq_length, head_size, stream, hidden);
+                                          heads, seq_length, head_size, stream, hidden, scale);
 }
 
 extern "C" int cubert_attention_fused_f16(const cubert_half *q, const cubert_half *k, const cubert_half *v, int ld,

@@ -44,12 +44,12 @@ __device__ __forceinline__ int uniform_i8(const int8_t *__restrict__ p, int inde
 
 // Normalise the row held in x[][] and store it.  gamma/beta were loaded before
 // the reduction so their latency overlaps it.
-// With `split_row` the stored values also go out as two-term fp16 rows [hi | hi | lo] (hi = fp16(y), lo = fp16(y - hi),
-// clamped to the fp16 range), the token operand of a Dense GEMM on the fp16 matrix cores (see split.hip).
+// With `split_row` the stored values, times split_scale, also go out as two-term fp16 rows [hi | hi | lo] (hi = fp16(y),
+// lo = fp16(y - hi), clamped to the fp16 range), the token operand of a Dense GEMM on the fp16 matrix cores (see split.hip).
 template <typename T, int VEC, int CHUNKS>
 __device__ __forceinline__ void ln_finish(float (&x)[CHUNKS][VEC], float sum, float sumsq, const Vec<T, VEC> (&g)[CHUNKS],
                                           const Vec<T, VEC> (&b)[CHUNKS], T *__restrict__ out_row, int lane,
-                                          half_t *__restrict__ split_row = nullptr) {
+                                          half_t *__restrict__ split_row = nullptr, float split_scale = 1.f) {
     constexpr int H = kWave * VEC * CHUNKS;
     float mean, rstd;
     ln_stats(sum, sumsq, H, mean, rstd);
@@ -65,7 +65,7 @@ __device__ __forceinline__ void ln_finish(float (&x)[CHUNKS][VEC], float sum, fl
             Vec<half_t, VEC> hi, lo;
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
-                const float y = to_f32(o.v[i]);
+                const float y = to_f32(o.v[i]) * split_scale;
                 hi.v[i] = (half_t) fminf(fmaxf(y, -65504.f), 65504.f);
                 lo.v[i] = (half_t) fminf(fmaxf(y - (float) hi.v[i], -65504.f), 65504.f);
             }
@@ -81,7 +81,7 @@ template <typename T, int VEC, int CHUNKS, bool HAS_BIAS, bool SPLIT = false>
 __global__ __launch_bounds__(kBlock) void bias_res_ln_kernel(T *__restrict__ inout, const T *__restrict__ residual,
                                                              const T *__restrict__ bias, const T *__restrict__ beta,
                                                              const T *__restrict__ gamma, int rows,
-                                                             half_t *__restrict__ split_out) {
+                                                             half_t *__restrict__ split_out, float split_scale) {
     constexpr int H = kWave * VEC * CHUNKS;
     const int row = blockIdx.x * kRowsPerBlock + wave_in_block();
     if (row >= rows) return;
@@ -119,7 +119,8 @@ __global__ __launch_bounds__(kBlock) void bias_res_ln_kernel(T *__restrict__ ino
             sumsq += v * v;
         }
     }
-    ln_finish<T, VEC, CHUNKS>(x, sum, sumsq, g, be, io, lane, SPLIT ? split_out + (size_t) row * 3 * H : nullptr);
+    ln_finish<T, VEC, CHUNKS>(x, sum, sumsq, g, be, io, lane, SPLIT ? split_out + (size_t) row * 3 * H : nullptr,
+                              split_scale);
 }
 
 template <typename T, int VEC, int CHUNKS>
@@ -350,9 +351,9 @@ int bias_res_ln(T *inout, const T *residual, const T *bias, const T *beta, const
     if (hidden == kWave * VEC * CHUNKS && vector_ok<T>(hidden, VEC, {inout, residual, bias, beta, gamma})) { \
         if (bias != nullptr)                                                                             \
             return launch(bias_res_ln_kernel<T, VEC, CHUNKS, true>, grid, block, s, inout, residual, bias, beta, gamma, \
-                          rows, nullptr);                                                                \
+                          rows, nullptr, 1.f);                                                           \
         return launch(bias_res_ln_kernel<T, VEC, CHUNKS, false>, grid, block, s, inout, residual, bias, beta, gamma, \
-                      rows, nullptr);                                                                    \
+                      rows, nullptr, 1.f);                                                               \
     }
     CUBERT_LN_CASE(V, 1)
     CUBERT_LN_CASE(V, 2)
@@ -373,7 +374,7 @@ int bias_res_ln(T *inout, const T *residual, const T *bias, const T *beta, const
 // bias + residual + LayerNorm of fp32 rows, in place, and the result again as two-term fp16 rows in split_out
 // [rows, 3 * hidden]; only the register-resident shapes (hidden = 256 k), anything else is declined.
 int bias_res_ln_split3(float *inout, const float *residual, const float *bias, const float *beta, const float *gamma,
-                       int rows, int hidden, half_t *split_out, void *stream) {
+                       int rows, int hidden, float scale, half_t *split_out, void *stream) {
     if (rows < 0 || hidden <= 0 || !inout || !residual || !beta || !gamma || !split_out) return CUBERT_BAD_ARGUMENT;
     if (rows == 0) return 0;
     hipStream_t s = (hipStream_t) stream;
@@ -383,9 +384,9 @@ int bias_res_ln_split3(float *inout, const float *residual, const float *bias, c
     if (hidden == kWave * 4 * CHUNKS && vector_ok<float>(hidden, 4, {inout, residual, bias, beta, gamma})) {         \
         if (bias != nullptr)                                                                                          \
             return launch(bias_res_ln_kernel<float, 4, CHUNKS, true, true>, grid, block, s, inout, residual, bias, beta, \
-                          gamma, rows, split_out);                                                                    \
+                          gamma, rows, split_out, scale);                                                             \
         return launch(bias_res_ln_kernel<float, 4, CHUNKS, false, true>, grid, block, s, inout, residual, bias, beta,  \
-                      gamma, rows, split_out);                                                                        \
+                      gamma, rows, split_out, scale);                                                                 \
     }
     CUBERT_LN_SPLIT_CASE(1)
     CUBERT_LN_SPLIT_CASE(2)
@@ -448,10 +449,10 @@ extern "C" int cubert_bias_res_ln_f32(float *inout, const float *residual, const
 }
 
 extern "C" int cubert_bias_res_ln_split3_f32(float *inout, const float *residual, const float *bias, const float *beta,
-                                             const float *gamma, int rows, int hidden, cubert_half *split_out,
-                                             void *stream) {
-    return cubert::bias_res_ln_split3(inout, residual, bias, beta, gamma, rows, hidden, (cubert::half_t *) split_out,
-                                      stream);
+                                             const float *gamma, int rows, int hidden, float scale,
+                                             cubert_half *split_out, void *stream) {
+    return cubert::bias_res_ln_split3(inout, residual, bias, beta, gamma, rows, hidden, scale,
+                                      (cubert::half_t *) split_out, stream);
 }
 
 extern "C" int cubert_bias_res_ln_f16(cubert_half *inout, const cubert_half *residual, const cubert_half *bias,

@@ -9,10 +9,11 @@
 // The fp16 matrix-core rate of this part is 16 times its fp32 rate, so the threefold GEMM is still several times
 // faster (reference Dense: src/cuBERT/op/Dense.cpp:47-57, one fp32 GEMM).
 //
-// Range: fp16 holds |hi| <= 65504, and lo loses bits once it is subnormal (|x| < 2^-3 leaves an absolute error of up
-// to 2^-25; harmless for an activation row whose larger entries are of order 1).  Weights are scaled by a power of
-// two per matrix (passed in as `scale`, taken out again by the GEMM's alpha), so their size does not matter;
-// activations are taken as they are and clamped to the fp16 range.
+// Range: fp16 holds |hi| <= 65504, and lo loses bits once it is subnormal (a scaled value below 2^-3 leaves an
+// absolute error of up to 2^-25).  Both sides are therefore multiplied by a power of two before they are taken
+// apart (`scale`, exact, taken out again by the GEMM's alpha): weights per matrix, so that the largest is in
+// [512, 1024) and their size does not matter; activations by a fixed factor chosen by the caller (the host classes
+// use 16: full accuracy for rows whose entries are of order 2^-7 to 2^12), clamped to the fp16 range beyond it.
 
 #include "cubert_kernels.h"
 #include "activations.h"
@@ -31,7 +32,7 @@ __device__ __forceinline__ void split_two(float x, half_t &hi, half_t &lo) {
     lo = (half_t) fminf(fmaxf(x - (float) hi, -kMax), kMax);
 }
 
-// out[row] = [hi | hi | lo] (LO_IN_MIDDLE: [hi | lo | hi]) of f(scale * in[row] + bias), each part `width` halves.
+// out[row] = [hi | hi | lo] (LO_IN_MIDDLE: [hi | lo | hi]) of scale * f(in[row] + bias), each part `width` halves.
 // One workgroup per row, threads walk the columns 8 at a time: two 16-byte loads, three 16-byte stores.
 template <typename Op, bool LO_IN_MIDDLE>
 __global__ __launch_bounds__(kBlock) void split3_kernel(const float *__restrict__ in, const float *__restrict__ bias,
@@ -49,8 +50,8 @@ __global__ __launch_bounds__(kBlock) void split3_kernel(const float *__restrict_
         Vec<half_t, 8> hi, lo;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            split_two(op(fmaf(x0.v[i], scale, b0.v[i])), hi.v[i], lo.v[i]);
-            split_two(op(fmaf(x1.v[i], scale, b1.v[i])), hi.v[4 + i], lo.v[4 + i]);
+            split_two(op(x0.v[i] + b0.v[i]) * scale, hi.v[i], lo.v[i]);
+            split_two(op(x1.v[i] + b1.v[i]) * scale, hi.v[4 + i], lo.v[4 + i]);
         }
         store_vec<half_t, 8>(dst + col, hi);
         store_vec<half_t, 8>(dst + width + col, LO_IN_MIDDLE ? lo : hi);
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(kBlock) void split3_scalar_kernel(const float *__re
     Op op;
     for (int col = threadIdx.x; col < width; col += blockDim.x) {
         half_t hi, lo;
-        split_two(op(fmaf(row[col], scale, bias != nullptr ? bias[col] : 0.f)), hi, lo);
+        split_two(op(row[col] + (bias != nullptr ? bias[col] : 0.f)) * scale, hi, lo);
         dst[col] = hi;
         dst[width + col] = LO_IN_MIDDLE ? lo : hi;
         dst[2 * width + col] = LO_IN_MIDDLE ? hi : lo;
@@ -98,8 +99,8 @@ extern "C" int cubert_split3_f32(const float *in, int rows, int width, float sca
                         : split3<IdentityOp, false>(in, nullptr, rows, width, scale, (half_t *) out, stream);
 }
 
-extern "C" int cubert_bias_gelu_split3_f32(const float *in, const float *bias, int rows, int width, cubert_half *out,
-                                           void *stream) {
+extern "C" int cubert_bias_gelu_split3_f32(const float *in, const float *bias, int rows, int width, float scale,
+                                           cubert_half *out, void *stream) {
     using namespace cubert;
-    return split3<GeluOp<float>, false>(in, bias, rows, width, 1.f, (half_t *) out, stream);
+    return split3<GeluOp<float>, false>(in, bias, rows, width, scale, (half_t *) out, stream);
 }

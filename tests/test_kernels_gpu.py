@@ -397,11 +397,11 @@ def test_bias_gelu_split3_against_oracle(K, rows, width):
     rng = np.random.default_rng(width)
     x = (rng.normal(0, 2, (rows, width))).astype(np.float32)
     b = rng.normal(0, 0.5, width).astype(np.float32)
-    got = K.bias_gelu_split3(dev(x), dev(b))
+    got = K.bias_gelu_split3(dev(x), dev(b), 16.0)
     torch.cuda.synchronize()
     got = got.cpu().numpy()
     assert np.array_equal(got[:, :width].view(np.uint16), got[:, width:2 * width].view(np.uint16))
-    value = got[:, :width].astype(np.float64) + got[:, 2 * width:].astype(np.float64)
+    value = (got[:, :width].astype(np.float64) + got[:, 2 * width:].astype(np.float64)) / 16
     want = oracle.gelu(x + b)
     assert_close(value, want, FP32_TOL, "two-term GELU")
     # and against the in-place kernel, to the resolution of the two terms
@@ -419,9 +419,9 @@ def test_bias_res_ln_split3_equals_ln_then_split(K, rows, hidden, with_bias):
     gamma = rng.normal(1, 0.1, hidden).astype(np.float32)
     args = [dev(res), None if bias is None else dev(bias), dev(beta), dev(gamma)]
     plain = K.bias_res_ln_(dev(x), *args)
-    want_split = K.split3(plain)
+    want_split = K.split3(plain, 16.0)
     inout = dev(x)
-    got_split = K.bias_res_ln_split3_(inout, *args)
+    got_split = K.bias_res_ln_split3_(inout, *args, scale=16.0)
     assert got_split is not None
     torch.cuda.synchronize()
     assert torch.equal(inout, plain)             # the fp32 result is the plain kernel's, bit for bit
@@ -441,10 +441,10 @@ def test_attention_fused_split3_equals_attention_then_split(K, batch, heads, seq
     alpha = 1.0 / math.sqrt(d)
     plain = K.attention_fused(qkv, mask, batch, heads, seq, d, alpha)
     assert plain is not None
-    got = K.attention_fused_split3(qkv, mask, batch, heads, seq, d, alpha)
+    got = K.attention_fused_split3(qkv, mask, batch, heads, seq, d, alpha, scale=16.0)
     assert got is not None
     torch.cuda.synchronize()
-    assert torch.equal(got, K.split3(plain))  # the same context values, written in the other form
+    assert torch.equal(got, K.split3(plain, 16.0))  # the same context values, written in the other form
 
 
 def test_bias_res_ln_split3_declines_other_hidden_sizes(K):
