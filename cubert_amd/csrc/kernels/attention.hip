@@ -22,6 +22,7 @@
 //     consecutive k for a fixed column and V is stored with consecutive columns.
 
 #include <atomic>
+#include <cstdlib>
 #include <initializer_list>
 
 #include "cubert_kernels.h"
@@ -797,6 +798,237 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
     }
 }
 
+// ---- seq 512 with the keys staged a group at a time ----
+// attention_flash_kernel keeps K and V of the whole head in LDS, which at seq 512 leaves room for one workgroup per
+// compute unit, so nothing overlaps its load, compute and store phases.  Here the 16 wavefronts of a workgroup walk
+// the live key tiles in groups of G = 32 V / D tiles (4 for fp16, head size 64): load a group (one K vector and one
+// V^T slot group per thread), barrier, online-softmax update from it, barrier, next group.  A quarter of the LDS:
+// two workgroups share a compute unit (the limit is then the 32 wavefronts, not the LDS) and the phases of one
+// overlap those of the other; fp32 at seq 512 fits as well.  Arithmetic and rounding are those of
+// attention_flash_kernel.
+template <typename T, int D, bool SPLIT>
+__global__ __launch_bounds__(1024) void attention_flash_grouped_kernel(
+    const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, int ld, const int8_t *__restrict__ mask,
+    T *__restrict__ ctx, int ld_ctx, float alpha, int heads, int skip_masked_tiles, int split_width, float split_scale) {
+    constexpr int V = Mma<T>::kVec;
+    constexpr int kSteps = D / 2 / V;
+    constexpr int kColTiles = D / 32;
+    constexpr int kChunk = 2;                // key tiles per online-softmax step
+    constexpr int G = 32 * V / D;            // key tiles per group
+    constexpr int kThreads = 1024;
+    constexpr int kSeq = 512;
+    constexpr int kPitchK = D + V;
+    constexpr int kPitchV = G * 32 + V;
+    constexpr int kVecPerRow = D / V;
+    constexpr int kLoads = G * 32 * kVecPerRow / kThreads;  // = 1: vectors per thread for K, slot groups for V^T
+    static_assert(kLoads == 1, "one K vector and one V^T slot group per thread");
+    constexpr int S = kSeq, KT = kSeq / 32;
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *s_k = reinterpret_cast<T *>(smem);                                      // [G * 32][kPitchK]
+    T *s_vt = s_k + G * 32 * kPitchK;                                          // [D][kPitchV], keys in slot order
+    float *s_mask = reinterpret_cast<float *>(s_vt + D * kPitchV);             // [S] additive mask
+    float *s_factor = s_mask + S;                                              // [16][32] per-query factors
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int r = lane & 31, hh = lane >> 5;
+    const int wave = wave_in_block();
+    const int bh = blockIdx.x;
+    const int b = bh / heads, h = bh - b * heads;
+    const int qt = wave;
+    const T *k_head = k + (size_t) b * S * ld + (size_t) h * D;
+    const T *v_head = v + (size_t) b * S * ld + (size_t) h * D;
+
+    const T *q_row = q + ((size_t) b * S + qt * 32 + r) * ld + (size_t) h * D + hh * (D / 2);
+    Vec<T, V> qv[kSteps];
+#pragma unroll
+    for (int t = 0; t < kSteps; ++t) qv[t] = load_vec<T, V>(q_row + t * V);
+
+    // bit kt: key tile kt has an unmasked key (workgroup-uniform: scalar loads of the mask row as words)
+    unsigned live = 0;
+    if (mask != nullptr && skip_masked_tiles) {
+        const uint32_t *words = reinterpret_cast<const uint32_t *>(mask + (size_t) b * S);
+        for (int kt = 0; kt < KT; ++kt) {
+            uint32_t any = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) any |= words[kt * 8 + i];
+            live |= (any != 0 ? 1u : 0u) << kt;
+        }
+    }
+    if (live == 0) live = KT >= 32 ? ~0u : (1u << KT) - 1u;
+    live = __builtin_amdgcn_readfirstlane(live);
+
+    for (int i = threadIdx.x; i < S; i += kThreads) {
+        s_mask[i] = (mask != nullptr && !mask[(size_t) b * S + i]) ? kMaskedScore * kLog2e : 0.f;
+    }
+
+    const float scale = alpha * kLog2e;
+    float *factor = s_factor + wave * 32;  // private to this wavefront
+    float m = -3.402823466e+38f, l = 0.f;
+    v16f32 out[kColTiles];
+#pragma unroll
+    for (int jt = 0; jt < kColTiles; ++jt) out[jt] = v16f32{};
+    bool first_chunk = true;
+
+    for (unsigned todo = live; todo != 0;) {
+        // the next group: the lowest G live tiles that are left
+        unsigned group = 0;
+        for (int i = 0; i < G && todo != 0; ++i) {
+            const unsigned low = todo & (0u - todo);
+            group |= low;
+            todo ^= low;
+        }
+        const int in_group = __builtin_popcount(group);
+        // tile of slot s: the s-th set bit of group (wavefront-uniform: a wavefront's 64 vectors lie in one tile)
+        auto tile_of = [&](int slot) {
+            unsigned rest = group;
+            for (int i = 0; i < slot; ++i) rest &= rest - 1;
+            return __builtin_ctz(rest);
+        };
+        Vec<T, V> kreg[kLoads], vreg[kLoads];
+#pragma unroll
+        for (int u = 0; u < kLoads; ++u) {
+            const int idx = threadIdx.x + u * kThreads;
+            const int slot = idx / (32 * kVecPerRow), within = idx - slot * (32 * kVecPerRow);
+            const int row = within / kVecPerRow, c = within - row * kVecPerRow;
+            kreg[u] = Vec<T, V>{};
+            if (slot < in_group) kreg[u] = load_vec<T, V>(k_head + (size_t) (tile_of(slot) * 32 + row) * ld + c * V);
+        }
+#pragma unroll
+        for (int u = 0; u < kLoads; ++u) {
+            const int idx = threadIdx.x + u * kThreads;
+            const int j = idx % D, grp = idx / D;               // grp: slot group of V keys, (32 / V) per tile
+            const int slot = grp / (32 / V), in_tile = grp % (32 / V);
+            const int run = in_tile >> 1, half = in_tile & 1;
+            vreg[u] = Vec<T, V>{};
+            if (slot < in_group) {
+                const int kt = tile_of(slot);
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    vreg[u].v[e] = v_head[(size_t) (kt * 32 + acc_row(run * V + e, half)) * ld + j];
+                }
+            }
+        }
+        __syncthreads();  // everyone is done with the previous group's tiles
+#pragma unroll
+        for (int u = 0; u < kLoads; ++u) {
+            const int idx = threadIdx.x + u * kThreads;
+            const int row = idx / kVecPerRow, c = idx - row * kVecPerRow;  // row = slot * 32 + row in tile
+            store_vec<T, V>(s_k + row * kPitchK + c * V, kreg[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kLoads; ++u) {
+            const int idx = threadIdx.x + u * kThreads;
+            const int j = idx % D, grp = idx / D;
+            store_vec<T, V>(s_vt + j * kPitchV + grp * V, vreg[u]);
+        }
+        __syncthreads();
+        int slot0 = 0;
+        for (unsigned rest = group; rest != 0;) {  // the group's tiles in ascending order, kChunk per step
+            int tiles[kChunk], slots[kChunk];
+#pragma unroll
+            for (int cc = 0; cc < kChunk; ++cc) {
+                tiles[cc] = -1;
+                slots[cc] = 0;
+                if (rest != 0) {
+                    tiles[cc] = __builtin_ctz(rest);
+                    slots[cc] = slot0++;
+                    rest &= rest - 1;
+                }
+            }
+            v16f32 p[kChunk];
+            float cm = -3.402823466e+38f;
+#pragma unroll
+            for (int cc = 0; cc < kChunk; ++cc) {
+                v16f32 c = {};
+                if (tiles[cc] >= 0) {  // wavefront-uniform
+#pragma unroll
+                    for (int t = 0; t < kSteps; ++t) {
+                        Mma<T>::run(c, load_vec<T, V>(s_k + (slots[cc] * 32 + r) * kPitchK + hh * (D / 2) + t * V), qv[t]);
+                    }
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const Vec<float, 4> mk = load_vec<float, 4>(s_mask + tiles[cc] * 32 + g * 8 + hh * 4);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float sc = fmaf(c[g * 4 + e], scale, mk.v[e]);
+                            c[g * 4 + e] = sc;
+                            cm = fmaxf(cm, sc);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) c[i] = -3.402823466e+38f;  // exp(. - m) = 0
+                }
+                p[cc] = c;
+            }
+            cm = fmaxf(cm, __shfl_xor(cm, 32, kWave));
+            const float m_new = fmaxf(m, cm);
+            const float f = __builtin_amdgcn_exp2f(m - m_new);
+            float part = 0.f;
+#pragma unroll
+            for (int cc = 0; cc < kChunk; ++cc) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    p[cc][i] = __builtin_amdgcn_exp2f(p[cc][i] - m_new);
+                    part += p[cc][i];
+                }
+            }
+            part += __shfl_xor(part, 32, kWave);
+            l = l * f + part;
+            m = m_new;
+            if (!first_chunk && __any(f != 1.f)) {  // wavefront-uniform: skipped when no query's maximum moved
+                if (hh == 0) factor[r] = f;
+                __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): LDS operations of one wavefront complete in order
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const Vec<float, 4> fr = load_vec<float, 4>(factor + g * 8 + hh * 4);
+#pragma unroll
+                    for (int jt = 0; jt < kColTiles; ++jt) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) out[jt][g * 4 + e] *= fr.v[e];
+                    }
+                }
+                __builtin_amdgcn_wave_barrier();  // the reads above come before the next chunk's write
+            }
+            first_chunk = false;
+#pragma unroll
+            for (int cc = 0; cc < kChunk; ++cc) {
+                if (tiles[cc] >= 0) {
+#pragma unroll
+                    for (int run = 0; run < 16 / V; ++run) {
+                        Vec<T, V> a;
+#pragma unroll
+                        for (int e = 0; e < V; ++e) a.v[e] = from_f32<T>(p[cc][run * V + e]);
+#pragma unroll
+                        for (int jt = 0; jt < kColTiles; ++jt) {
+                            Mma<T>::run(out[jt], a,
+                                        load_vec<T, V>(s_vt + (jt * 32 + r) * kPitchV + slots[cc] * 32 + run * 2 * V + hh * V));
+                        }
+                    }
+                }
+            }
+        }
+    }
+    // divide row (query) i by its sum
+    if (hh == 0) factor[r] = 1.f / l;
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_wave_barrier();
+    const size_t first_row = (size_t) b * S + qt * 32;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const Vec<float, 4> fr = load_vec<float, 4>(factor + g * 8 + hh * 4);
+#pragma unroll
+        for (int jt = 0; jt < kColTiles; ++jt) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                store_context<T, SPLIT>(ctx, ld_ctx, first_row + acc_row(g * 4 + e, hh), h * D + jt * 32 + r,
+                                        out[jt][g * 4 + e] * fr.v[e], split_width, split_scale);
+            }
+        }
+    }
+}
+
 template <typename T>
 bool shapes_ok(int batch, int heads, int seq, int head_size, int ld, std::initializer_list<const void *> ptrs) {
     constexpr int V = Mma<T>::kVec;
@@ -959,8 +1191,25 @@ int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask,
     if (seq > 512) return CUBERT_UNSUPPORTED;  // a workgroup has at most 16 wavefronts
     const size_t lds = (size_t) seq * (D + V) * sizeof(T) + (size_t) D * (seq + V) * sizeof(T) +
                        2 * (size_t) seq * sizeof(float);
-    if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
     const int skip_masked_tiles = mask != nullptr && is_aligned(mask, 4);  // seq is a multiple of 32
+    static const bool whole_head = getenv("CUBERT_FLASH_WHOLE") != nullptr;
+    if (seq == 512 && !whole_head) {
+        constexpr int G = 32 * V / D;
+        const size_t grouped_lds = ((size_t) G * 32 * (D + V) + (size_t) D * (G * 32 + V)) * sizeof(T) +
+                                   ((size_t) seq + 16 * 32) * sizeof(float);
+        if constexpr (sizeof(T) == 4) {
+            if (split_width > 0) {
+                return launch_untimed(attention_flash_grouped_kernel<T, D, true>, dim3(batch * heads), dim3(1024),
+                                      (unsigned) grouped_lds, s, q, k, v, ld, mask, ctx, ld_ctx, alpha, heads,
+                                      skip_masked_tiles, split_width, split_scale);
+            }
+        }
+        if (split_width > 0) return CUBERT_UNSUPPORTED;
+        return launch_untimed(attention_flash_grouped_kernel<T, D, false>, dim3(batch * heads), dim3(1024),
+                              (unsigned) grouped_lds, s, q, k, v, ld, mask, ctx, ld_ctx, alpha, heads, skip_masked_tiles,
+                              split_width, split_scale);
+    }
+    if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
     if constexpr (sizeof(T) == 4) {
         if (split_width > 0) {
             auto kernel = attention_flash_kernel<T, D, true>;

@@ -430,7 +430,7 @@ def test_bias_res_ln_split3_equals_ln_then_split(K, rows, hidden, with_bias):
 
 
 @pytest.mark.parametrize("batch,heads,seq,d", [(1, 12, 32, 64), (24, 12, 32, 64), (3, 4, 128, 64), (2, 3, 64, 32),
-                                               (1, 2, 256, 64), (2, 2, 96, 128)])
+                                               (1, 2, 256, 64), (2, 2, 96, 128), (1, 2, 512, 64)])
 def test_attention_fused_split3_equals_attention_then_split(K, batch, heads, seq, d):
     rng = np.random.default_rng(batch + heads + seq + d)
     H = heads * d
@@ -520,8 +520,10 @@ def test_attention_scores_and_context(K, name, batch, heads, seq, d):
                                                # seq 32, head size 64: four wavefronts per problem up to 256
                                                # problems (above), one wavefront per problem beyond (below)
                                                (1, 12, 32, 64), (24, 12, 32, 64), (2, 2, 32, 32),
-                                               # longer than 128: the online-softmax kernel (chunks of 64 keys)
-                                               (1, 2, 512, 64), (2, 3, 256, 64), (2, 2, 160, 64), (1, 1, 384, 32)])
+                                               # longer than 128: the online-softmax kernels (chunks of 64 keys;
+                                               # seq 512 stages the keys in groups, the others the whole head)
+                                               (1, 2, 512, 64), (2, 3, 256, 64), (2, 2, 160, 64), (1, 1, 384, 32),
+                                               (2, 3, 512, 32)])
 @pytest.mark.parametrize("masked", [True, False])
 def test_attention_fused_against_oracle(K, name, batch, heads, seq, d, masked):
     """One-launch attention core vs the oracle's attention_self pieces (att_q_k -> mask -> softmax -> att_qk_v),
@@ -534,8 +536,8 @@ def test_attention_fused_against_oracle(K, name, batch, heads, seq, d, masked):
     mask[0, :] = 0
     alpha = 1.0 / math.sqrt(d)
     ctx = K.attention_fused(dev(qkv, tdt(name)), dev(mask) if masked else None, batch, heads, seq, d, alpha)
-    if ctx is None:  # K and V of one head must fit 160 KB of LDS
-        assert seq * (d + 4) * 4 + d * (seq + 4) * 4 + 2 * seq * 4 > 160 * 1024 and name == "f32"
+    if ctx is None:  # K and V of one head must fit 160 KB of LDS, except at seq 512 (keys staged in groups)
+        assert seq * (d + 4) * 4 + d * (seq + 4) * 4 + 2 * seq * 4 > 160 * 1024 and name == "f32" and seq != 512
         return
     scores = oracle.att_q_k(qh, kh, batch, seq, heads, d, alpha=alpha)  # [B, S_q, A, S_k]
     if name == "f16":
@@ -564,7 +566,7 @@ def test_attention_fused_against_oracle(K, name, batch, heads, seq, d, masked):
 
 
 @pytest.mark.parametrize("name", ["f32", "f16"])
-@pytest.mark.parametrize("heads,seq,d", [(2, 512, 64), (3, 256, 64), (2, 160, 64), (1, 384, 32)])
+@pytest.mark.parametrize("heads,seq,d", [(2, 512, 64), (3, 256, 64), (2, 160, 64), (1, 384, 32), (2, 512, 32)])
 def test_attention_long_sequences_with_padding(K, name, heads, seq, d):
     """The online-softmax kernel leaves out key tiles (32 keys) that are masked throughout.  Masks with whole tiles
     of zeros in every position (prefix padding, live tiles scattered between dead ones, a single unmasked key in
@@ -573,7 +575,7 @@ def test_attention_long_sequences_with_padding(K, name, heads, seq, d):
     batch = 6
     rng = np.random.default_rng(heads * 100 + seq + d)
     H = heads * d
-    if name == "f32" and seq * (d + 4) * 4 + d * (seq + 4) * 4 + 2 * seq * 4 > 160 * 1024:
+    if name == "f32" and seq != 512 and seq * (d + 4) * 4 + d * (seq + 4) * 4 + 2 * seq * 4 > 160 * 1024:
         pytest.skip("K and V of one head do not fit the LDS in fp32")
     qkv = q(rng.normal(0, 1, (batch * seq, 3 * H)), name)
     qh, kh, vh = (np.ascontiguousarray(x) for x in (qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:]))
@@ -731,7 +733,29 @@ def test_empty_and_bad_arguments(K):
     assert L.cubert_bias_gelu_f32(x.data_ptr(), None, 4, 0, None) == -1
     assert L.cubert_mask_scale_softmax_f32(x.data_ptr(), None, 1.0, 1, 0, 32, None) == -1
     assert L.cubert_mean_pool_f32(x.data_ptr(), x.data_ptr(), 1, 0, 768, None) == -1
+    # the two-term operand kernels
+    h = torch.zeros((4, 3 * 768), dtype=torch.float16, device="cuda")
+    assert L.cubert_split3_f32(x.data_ptr(), 0, 768, 1.0, 0, h.data_ptr(), None) == 0
+    assert L.cubert_split3_f32(x.data_ptr(), 4, 0, 1.0, 0, h.data_ptr(), None) == -1
+    assert L.cubert_split3_f32(None, 4, 768, 1.0, 0, h.data_ptr(), None) == -1
+    assert L.cubert_bias_gelu_split3_f32(x.data_ptr(), None, 0, 768, 1.0, h.data_ptr(), None) == 0
+    assert L.cubert_bias_gelu_split3_f32(x.data_ptr(), None, 4, 768, 1.0, None, None) == -1
+    assert L.cubert_bias_res_ln_split3_f32(x.data_ptr(), x.data_ptr(), None, x.data_ptr(), x.data_ptr(), 0, 768, 1.0,
+                                           h.data_ptr(), None) == 0
+    assert L.cubert_bias_res_ln_split3_f32(x.data_ptr(), x.data_ptr(), None, x.data_ptr(), x.data_ptr(), 4, 768, 1.0,
+                                           None, None) == -1
     torch.cuda.synchronize()
+
+
+def test_split3_unaligned_and_odd_widths_take_the_generic_path(K):
+    rng = np.random.default_rng(11)
+    base = torch.zeros(5 * 24 + 1, device="cuda")
+    x = rng.normal(0, 1, (5, 24)).astype(np.float32)
+    base[1:] = dev(x).reshape(-1)
+    view = base[1:].view(5, 24)          # 4-byte aligned only
+    assert torch.equal(K.split3(view, 2.0), K.split3(dev(x), 2.0))
+    b = dev(rng.normal(0, 1, 24).astype(np.float32))
+    assert torch.equal(K.bias_gelu_split3(view, b, 16.0), K.bias_gelu_split3(dev(x), b, 16.0))
 
 
 def test_unaligned_views_take_the_generic_path(K):
