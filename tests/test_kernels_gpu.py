@@ -453,13 +453,16 @@ def test_bias_res_ln_split3_declines_other_hidden_sizes(K):
     assert K.bias_res_ln_split3_(x, x.clone(), None, v, v) is None
 
 
-@pytest.mark.parametrize("tokens,in_features,out_features", [(4096, 768, 2304), (200, 3072, 768), (64, 128, 512),
-                                                             (33, 40, 24)])
-def test_two_term_dense_matches_fp32_dense(K, tokens, in_features, out_features):
+@pytest.mark.parametrize("tokens,in_features,out_features,magnitude", [(4096, 768, 2304, 1.0), (200, 3072, 768, 1.0),
+                                                                       (64, 128, 512, 1.0), (33, 40, 24, 1.0),
+                                                                       # the ends of the range the host classes'
+                                                                       # activation scale of 16 is meant for
+                                                                       (256, 768, 768, 0.01), (256, 768, 768, 500.0)])
+def test_two_term_dense_matches_fp32_dense(K, tokens, in_features, out_features, magnitude):
     """Dense(x) = x W + b with both operands in two-term fp16 form on the mixed GEMM, against float64 and against
     the fp32 GEMM: the error of the form is that of fp32 arithmetic (accumulation rounding dominates both)."""
     rng = np.random.default_rng(tokens + in_features)
-    x = rng.normal(0, 1, (tokens, in_features)).astype(np.float32)
+    x = (rng.normal(0, 1, (tokens, in_features)) * magnitude).astype(np.float32)
     w = rng.normal(0, 0.02, (in_features, out_features)).astype(np.float32)
     b = rng.normal(0, 0.02, out_features).astype(np.float32)
     want = x.astype(np.float64) @ w.astype(np.float64) + b
@@ -470,9 +473,9 @@ def test_two_term_dense_matches_fp32_dense(K, tokens, in_features, out_features)
               out_features, db)
     exponent = 10 - math.frexp(float(np.abs(w).max()))[1]
     w3 = K.split3(K.transpose(dw), 2.0 ** exponent, True)       # [out, 3 in]: hi | lo | hi
-    x3 = K.split3(dx)                                           # [tokens, 3 in]: hi | hi | lo
+    x3 = K.split3(dx, 16.0)                                     # [tokens, 3 in]: hi | hi | lo of 16 x
     out = torch.empty((tokens, out_features), dtype=torch.float32, device="cuda")
-    blas.gemm_f16_f32(True, False, out_features, tokens, 3 * in_features, 2.0 ** -exponent, w3, 3 * in_features, x3,
+    blas.gemm_f16_f32(True, False, out_features, tokens, 3 * in_features, 2.0 ** -exponent / 16, w3, 3 * in_features, x3,
                       3 * in_features, 0.0, out, out_features, db)
     plain, out = host(plain), host(out)
     blas.close()
