@@ -158,3 +158,36 @@ def test_open_rejects_files_whose_tensors_do_not_fit_the_model(tmp_path):
             open_(w)
     else:
         open_(w)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """This build measures one GPU: `bench.py --gpus N` with N > 1 exits with a message instead of a number."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_bench_algorithmic_bytes_follow_the_published_formulas():
+    """Per-launch algorithmic bytes of the fused kernels at the benchmark shapes (every operand once)."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    from cubert_amd.testing import CONFIGS
+    os.environ.pop("CUBERT_FP32_DENSE", None)
+    mb = {name: {k: v / 1e6 for k, v in bench.algorithmic_bytes(CONFIGS[name]).items()} for name in CONFIGS}
+    # bias+GELU 2*M*I*e + I*e, bias+residual+LN 3*M*H*e + 3*H*e, mask+softmax 2*B*A*S^2*e + B*S, embed+LN
+    for name, gelu, ln, softmax, embed in (("C1", 100.7, 37.8, 12.6, 25.3), ("C3", 402.7, 151.0, 805.3, 101.6),
+                                           ("C4", 536.9, 201.3, 268.5, 134.7)):
+        assert abs(mb[name]["bias_gelu"] - gelu) < 0.06 and abs(mb[name]["bias_res_ln"] - ln) < 0.06
+        assert abs(mb[name]["mask_scale_softmax"] - softmax) < 0.06 and abs(mb[name]["embed_ln"] - embed) < 0.06
+    os.environ["CUBERT_FP32_DENSE"] = "f16x3"
+    try:
+        two_term = bench.algorithmic_bytes(CONFIGS["C1"])
+        half_model = bench.algorithmic_bytes(CONFIGS["C3"])
+    finally:
+        del os.environ["CUBERT_FP32_DENSE"]
+    assert two_term["bias_gelu"] == 4096 * 3072 * 10 + 3072 * 4 and two_term["dense_split"] == 4096 * 768 * 10
+    assert half_model["bias_gelu"] == bench.algorithmic_bytes(CONFIGS["C3"])["bias_gelu"]  # fp16 models: unchanged
