@@ -45,6 +45,10 @@ Transformer<T>::Transformer(void *cublas, const std::string &var_prefix,
     // Half-precision models therefore keep their Dense kernels [out, in], transposed once here.
     transposed_kernels = sizeof(T) == 2;
     const char *dense_mode = std::getenv("CUBERT_FP32_DENSE");
+    if (dense_mode != nullptr && std::string(dense_mode) != "f16x3" && std::string(dense_mode) != "f32" &&
+        std::string(dense_mode) != "") {
+        fprintf(stderr, "cuBERT: CUBERT_FP32_DENSE=%s is not understood (f32 or f16x3); using f32\n", dense_mode);
+    }
     split_dense = sizeof(T) == 4 && dense_mode != nullptr && std::string(dense_mode) == "f16x3" &&
                   max_batch_size * seq_length >= kTwoTermMinTokens;
 
