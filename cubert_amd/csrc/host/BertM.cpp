@@ -1,6 +1,7 @@
 #include "BertM.h"
 
 #include <chrono>
+#include <cstdlib>
 #include <iostream>
 #include <stdexcept>
 #include <string>
@@ -65,7 +66,21 @@ BertM<T>::BertM(const char *model_file, size_t max_batch_size, size_t seq_length
     }
     std::cerr << "Found GPU count: " << count << std::endl;
 
-    for (int device = 0; device < count; ++device) {
+    // CUBERT_MODELS_PER_GPU=n in the environment (default 1) keeps n instances per device, each with its own stream:
+    // requests of a few tokens leave most of the chip idle (their kernels wait on memory latency), so concurrent
+    // callers get more requests per second when they do not queue behind one instance per device.  (The reference
+    // has the same knob for its CPU build, CUBERT_NUM_CPU_MODELS, src/cuBERT/BertM.cpp:25-28.)
+    int per_device = 1;
+    if (const char *text = std::getenv("CUBERT_MODELS_PER_GPU")) {
+        per_device = std::atoi(text);
+        if (per_device < 1 || count * per_device > 255) {
+            throw std::invalid_argument("CUBERT_MODELS_PER_GPU must be at least 1 and give at most 255 instances");
+        }
+        std::cerr << "Found CUBERT_MODELS_PER_GPU: " << per_device << std::endl;
+    }
+
+    for (int instance = 0; instance < count * per_device; ++instance) {
+        const int device = instance % count;  // round-robin over instances visits the devices in turn
         const auto start = std::chrono::high_resolution_clock::now();
         cuBERT::set_gpu(device);
         cuBERT::gpu_info(device);
@@ -73,6 +88,7 @@ BertM<T>::BertM(const char *model_file, size_t max_batch_size, size_t seq_length
                                                 graph.type_vocab_size, graph.hidden_size, num_hidden_layers,
                                                 num_attention_heads, graph.intermediate_size, graph.num_labels));
         mutex_instances.emplace_back(new std::mutex());
+        device_of_instance.push_back(device);
         const auto finish = std::chrono::high_resolution_clock::now();
         std::cerr << "device setup: " << device << ". Took "
                   << std::chrono::duration_cast<std::chrono::milliseconds>(finish - start).count() << " milliseconds."
@@ -83,7 +99,7 @@ BertM<T>::BertM(const char *model_file, size_t max_batch_size, size_t seq_length
 template <typename T>
 BertM<T>::~BertM() {
     for (size_t i = 0; i < bert_instances.size(); ++i) {
-        cuBERT::set_gpu((int) i);
+        cuBERT::set_gpu(device_of_instance[i]);
         bert_instances[i].reset();
     }
 }
@@ -94,7 +110,7 @@ unsigned int BertM<T>::compute(size_t batch_size, int *input_ids, int8_t *input_
     const uint8_t count = rr++;
     const unsigned int choice = count % bert_instances.size();
 
-    cuBERT::set_gpu((int) choice);
+    cuBERT::set_gpu(device_of_instance[choice]);
     Bert<T> *bert = bert_instances[choice].get();
     std::lock_guard<std::mutex> lg(*mutex_instances[choice]);
 
@@ -116,7 +132,7 @@ unsigned int BertM<T>::compute(size_t batch_size, int *input_ids, int8_t *input_
     const uint8_t count = rr++;
     const unsigned int choice = count % bert_instances.size();
 
-    cuBERT::set_gpu((int) choice);
+    cuBERT::set_gpu(device_of_instance[choice]);
     Bert<T> *bert = bert_instances[choice].get();
     std::lock_guard<std::mutex> lg(*mutex_instances[choice]);
 

@@ -1,7 +1,9 @@
 // A loaded model replicated on every visible GPU, safe to call from many host
 // threads: requests go round-robin over the replicas and hold that replica's
 // mutex for the whole compute + copy-out.  Public surface of the reference's
-// BertM<T> (src/cuBERT/BertM.h:17-37).
+// BertM<T> (src/cuBERT/BertM.h:17-37).  CUBERT_MODELS_PER_GPU=n in the environment
+// keeps n replicas per device (own weights, buffers and stream each), which
+// lets small concurrent requests overlap on one device.
 #ifndef CUBERT_HOST_BERTM_H
 #define CUBERT_HOST_BERTM_H
 
@@ -44,6 +46,7 @@ private:
     // owned: a constructor that throws half way (a later device fails) releases the replicas built so far
     std::vector<std::unique_ptr<Bert<T>>> bert_instances;
     std::vector<std::unique_ptr<std::mutex>> mutex_instances;
+    std::vector<int> device_of_instance;  // instance i runs on device i % gpu_count (CUBERT_MODELS_PER_GPU instances each)
     std::atomic<uint8_t> rr;
 };
 

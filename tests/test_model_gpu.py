@@ -355,6 +355,14 @@ def test_tokenize_compute(cb, small_pb, tmp_path):
     plain.close()
 
 
+def test_models_per_gpu_must_be_a_sane_count(cb, small_pb, monkeypatch):
+    path, _ = small_pb
+    for bad in ("0", "-2", "1000", "x"):
+        monkeypatch.setenv("CUBERT_MODELS_PER_GPU", bad)
+        with pytest.raises(ValueError):
+            cb.Model(path, 4, 32, 3, 4)
+
+
 def test_api_error_behaviour(cb, small_pb):
     path, _ = small_pb
     with pytest.raises(ValueError, match="model file not found"):
@@ -377,11 +385,15 @@ def test_api_error_behaviour(cb, small_pb):
     model.close()
 
 
-def test_concurrent_callers_share_one_model(cb, small_pb):
-    """cuBERT_compute is thread-safe per handle (one mutex per replica held for compute + copy-out)."""
+@pytest.mark.parametrize("models_per_gpu", [None, "3"])
+def test_concurrent_callers_share_one_model(cb, small_pb, monkeypatch, models_per_gpu):
+    """cuBERT_compute is thread-safe per handle (one mutex per replica held for compute + copy-out), with one
+    replica per device and with CUBERT_MODELS_PER_GPU replicas (requests then overlap on the device)."""
     import threading
     from cubert_amd.testing import random_inputs
     path, w = small_pb
+    if models_per_gpu is not None:
+        monkeypatch.setenv("CUBERT_MODELS_PER_GPU", models_per_gpu)
     model = cb.Model(path, 4, 32, 3, 4)
     cases = [random_inputs(seed=20 + i, batch=1 + i % 4, seq_length=32, vocab=SMALL["vocab"], min_valid=2)
              for i in range(8)]
