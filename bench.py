@@ -169,6 +169,10 @@ def main():
                     help="skip the extra leg that repeats the steps with CUBERT_FP32_DENSE=f16x3 (fp32 workloads)")
     ap.add_argument("--device-only", action="store_true",
                     help="only the device-resident steps (no host-path / batch-1 latency loops): for profiler runs")
+    ap.add_argument("--instances", type=int, default=0,
+                    help="extra leg: this many model instances on the GPU, one caller thread each, every caller sending "
+                         "the workload's batch through the host path (what CUBERT_MODELS_PER_GPU gives concurrent "
+                         "callers of cuBERT_compute); reported as `concurrent_instances`")
     ap.add_argument("--fp32-dense", choices=["f32", "f16x3"], default=None,
                     help="f16x3: open the model with CUBERT_FP32_DENSE=f16x3 (the opt-in two-term fp16 Dense form of fp32 "
                          "models); default: whatever the environment says, normally the fp32 GEMM")
@@ -306,6 +310,40 @@ def main():
                     "dtype": "f32 storage and accumulation; Dense products as three f16 matrix-core products of two-term "
                              "operands (CUBERT_FP32_DENSE=f16x3, opt-in)"}
 
+    # ---- several instances on the one GPU, one caller thread each (host arrays in, pooled output out)
+    concurrent = None
+    if args.instances > 0:
+        import threading
+        berts = [cubert_amd.Bert(w, B, S, m["layers"], m["heads"], 1 if half else 0) for _ in range(args.instances)]
+        calls = max(50, args.steps)
+
+        def caller(model, n, latencies):
+            o = cubert_amd.Output(np.empty((B, m["hidden"]), np.float16 if half else np.float32),
+                                  cubert_amd.OutputType.POOLED_OUTPUT)
+            for _ in range(n):
+                t = time.perf_counter()
+                model.compute(ids, mask, seg)
+                model.output(B, o)
+                latencies.append((time.perf_counter() - t) * 1e3)
+
+        for model in berts:
+            caller(model, 10, [])
+        lat = [[] for _ in berts]
+        threads = [threading.Thread(target=caller, args=(model, calls, lat[i])) for i, model in enumerate(berts)]
+        t0 = time.perf_counter()
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        elapsed = time.perf_counter() - t0
+        for model in berts:
+            model.close()
+        every = np.concatenate([np.array(x) for x in lat])
+        concurrent = {"instances": args.instances, "callers": args.instances, "calls_per_caller": calls,
+                      "requests_per_s": round(args.instances * calls / elapsed, 1),
+                      "sequences_per_s": round(args.instances * calls * B / elapsed, 1),
+                      "p50_ms": round(float(np.median(every)), 3), "p99_ms": round(float(np.percentile(every, 99)), 3)}
+
     # ---- CPU baseline: the oracle (a port of the reference's CPU path) on this host's cores
     cpu = None
     if not args.no_cpu and not args.device_only:
@@ -361,6 +399,8 @@ def main():
         line["dtype"] = "f32 storage and accumulation; Dense products as three f16 matrix-core products of two-term operands"
     if two_term is not None:
         line["two_term_fp16_dense"] = two_term
+    if concurrent is not None:
+        line["concurrent_instances"] = concurrent
     if kernels:
         line["kernels"] = kernels
     print(json.dumps(line))
