@@ -73,10 +73,11 @@ __device__ __forceinline__ void store_context(T *ctx, int ld_ctx, size_t row, in
         asm volatile("" : "+v"(v));
         v *= split_scale;
         half_t *p = reinterpret_cast<half_t *>(ctx) + row * 3 * split_width + col;
-        const half_t hi = (half_t) fminf(fmaxf(v, -65504.f), 65504.f);
+        half_t hi, lo;
+        split_two_terms(v, hi, lo);
         p[0] = hi;
         p[split_width] = hi;
-        p[2 * split_width] = (half_t) fminf(fmaxf(v - (float) hi, -65504.f), 65504.f);
+        p[2 * split_width] = lo;
     } else {
         ctx[row * ld_ctx + col] = from_f32<T>(v);
     }

@@ -39,6 +39,14 @@ __device__ __forceinline__ float from_f32<float>(float x) { return x; }
 template <>
 __device__ __forceinline__ half_t from_f32<half_t>(float x) { return (half_t) x; }  // round to nearest even
 
+// An fp32 value as the sum of two fp16 numbers, hi = fp16(x) and lo = fp16(x - hi) (x - hi is exact in fp32), both
+// clamped to the fp16 range: the operand form of the fp32 Dense layers that run on the fp16 matrix cores.
+__device__ __forceinline__ void split_two_terms(float x, half_t &hi, half_t &lo) {
+    constexpr float kMax = 65504.f;
+    hi = (half_t) fminf(fmaxf(x, -kMax), kMax);
+    lo = (half_t) fminf(fmaxf(x - (float) hi, -kMax), kMax);
+}
+
 // Widest vector (in elements) that is at most 16 bytes.
 template <typename T>
 struct MaxVec {

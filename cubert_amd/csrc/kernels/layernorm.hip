@@ -65,9 +65,7 @@ __device__ __forceinline__ void ln_finish(float (&x)[CHUNKS][VEC], float sum, fl
             Vec<half_t, VEC> hi, lo;
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
-                const float y = to_f32(o.v[i]) * split_scale;
-                hi.v[i] = (half_t) fminf(fmaxf(y, -65504.f), 65504.f);
-                lo.v[i] = (half_t) fminf(fmaxf(y - (float) hi.v[i], -65504.f), 65504.f);
+                split_two_terms(to_f32(o.v[i]) * split_scale, hi.v[i], lo.v[i]);
             }
             half_t *at = split_row + (c * kWave + lane) * VEC;
             store_vec<half_t, VEC>(at, hi);

@@ -26,12 +26,6 @@ struct IdentityOp {
     __device__ __forceinline__ float operator()(float x) const { return x; }
 };
 
-__device__ __forceinline__ void split_two(float x, half_t &hi, half_t &lo) {
-    constexpr float kMax = 65504.f;
-    hi = (half_t) fminf(fmaxf(x, -kMax), kMax);
-    lo = (half_t) fminf(fmaxf(x - (float) hi, -kMax), kMax);
-}
-
 // out[row] = [hi | hi | lo] (LO_IN_MIDDLE: [hi | lo | hi]) of scale * f(in[row] + bias), each part `width` halves.
 // One workgroup per row, threads walk the columns 8 at a time: two 16-byte loads, three 16-byte stores.
 template <typename Op, bool LO_IN_MIDDLE>
@@ -50,8 +44,8 @@ __global__ __launch_bounds__(kBlock) void split3_kernel(const float *__restrict_
         Vec<half_t, 8> hi, lo;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            split_two(op(x0.v[i] + b0.v[i]) * scale, hi.v[i], lo.v[i]);
-            split_two(op(x1.v[i] + b1.v[i]) * scale, hi.v[4 + i], lo.v[4 + i]);
+            split_two_terms(op(x0.v[i] + b0.v[i]) * scale, hi.v[i], lo.v[i]);
+            split_two_terms(op(x1.v[i] + b1.v[i]) * scale, hi.v[4 + i], lo.v[4 + i]);
         }
         store_vec<half_t, 8>(dst + col, hi);
         store_vec<half_t, 8>(dst + width + col, LO_IN_MIDDLE ? lo : hi);
@@ -69,7 +63,7 @@ __global__ __launch_bounds__(kBlock) void split3_scalar_kernel(const float *__re
     Op op;
     for (int col = threadIdx.x; col < width; col += blockDim.x) {
         half_t hi, lo;
-        split_two(op(row[col] + (bias != nullptr ? bias[col] : 0.f)) * scale, hi, lo);
+        split_two_terms(op(row[col] + (bias != nullptr ? bias[col] : 0.f)) * scale, hi, lo);
         dst[col] = hi;
         dst[width + col] = LO_IN_MIDDLE ? lo : hi;
         dst[2 * width + col] = LO_IN_MIDDLE ? hi : lo;
