@@ -159,6 +159,51 @@ def nfd(text):
     return buf.value.decode("utf8")
 
 
+class Graph(object):
+    """The float / binary16 constants of a frozen GraphDef file as the library's loader sees them (the C++ class
+    Graph<T>, reference src/cuBERT/tensorflow/Graph.h:10-23).  CPU only."""
+
+    def __init__(self, model_file, compute_type=ComputeType.FLOAT):
+        self._h = None
+        self.compute_type = compute_type
+        handle = ctypes.c_void_p()
+        _raise(lib().cubert_graph_open(os.fsencode(model_file), compute_type, ctypes.byref(handle)))
+        self._h = handle
+        sizes = (ctypes.c_size_t * 5)()
+        _raise(lib().cubert_graph_sizes(handle, compute_type, sizes))
+        (self.vocab_size, self.type_vocab_size, self.hidden_size, self.intermediate_size,
+         self.num_labels) = (int(v) for v in sizes)
+
+    def __len__(self):
+        return int(lib().cubert_graph_count(self._h, self.compute_type))
+
+    def var(self, name):
+        """A copy of var[name] (flat) and its declared shape, or None for a name the graph does not hold."""
+        n = ctypes.c_size_t()
+        dims = (ctypes.c_longlong * 8)()
+        rank = ctypes.c_int()
+        ptr = lib().cubert_graph_var(self._h, self.compute_type, name.encode(), ctypes.byref(n), dims, 8,
+                                     ctypes.byref(rank))
+        if not ptr:
+            return None
+        dtype = np.float32 if self.compute_type == ComputeType.FLOAT else np.float16
+        data = np.empty(n.value, dtype)
+        if n.value:
+            ctypes.memmove(data.ctypes.data, ptr, data.nbytes)
+        return data, tuple(int(d) for d in dims[:min(rank.value, 8)])
+
+    def close(self):
+        if self._h is not None:
+            _raise(lib().cubert_graph_close(self._h, self.compute_type))
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class Model(object):
     """A model opened from a frozen GraphDef file (cuBERT_open), one replica per visible GPU; with a vocabulary
     file also the tokenizer (cuBERT_open_tokenizer), as python/cuBERT.pyx:116-139 of the reference."""

@@ -43,6 +43,13 @@ SIGNATURES = {
     "cubert_try_compute_m": (ci, [vp, ci, vp, vp, vp, ctypes.POINTER(cuBERT_Output), ci, ci]),
     "cubert_try_close": (ci, [vp, ci]),
     "cubert_model_info": (ci, [vp, ci, ctypes.POINTER(ci), ctypes.POINTER(ci), ctypes.POINTER(ci)]),
+    "cubert_check_input_range": (ci, [vp, vp, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t]),
+    "cubert_graph_open": (ci, [ctypes.c_char_p, ci, ctypes.POINTER(vp)]),
+    "cubert_graph_count": (cll, [vp, ci]),
+    "cubert_graph_var": (vp, [vp, ci, ctypes.c_char_p, ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(cll), ci,
+                              ctypes.POINTER(ci)]),
+    "cubert_graph_sizes": (ci, [vp, ci, ctypes.POINTER(ctypes.c_size_t)]),
+    "cubert_graph_close": (ci, [vp, ci]),
     "cubert_try_open_tokenizer": (ci, [ctypes.c_char_p, ci, ctypes.POINTER(vp)]),
     "cubert_try_tokenize_compute": (ci, [vp, vp, ci, vp, vp, vp, ci, ci]),
     "cubert_try_tokenize_compute_m": (ci, [vp, vp, ci, vp, vp, ctypes.POINTER(cuBERT_Output), ci, ci]),

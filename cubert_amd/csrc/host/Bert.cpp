@@ -13,12 +13,37 @@ inline size_t round_up_16(size_t n) { return (n + 15) & ~size_t(15); }
 inline size_t input_block_bytes(size_t M) { return round_up_16(round_up_16(sizeof(int) * M) + M) + M; }
 }  // namespace
 
+// Every id indexes a row of an embedding table on the device, where nothing checks it (nor does the reference,
+// src/cuBERT/op/Embedding.cpp:16-19): ids are checked here, on the host, before anything is enqueued.
+void check_input_range(const int *input_ids, const int8_t *segment_ids, size_t count, size_t vocab_size,
+                       size_t type_vocab_size) {
+    unsigned bad_id = 0, bad_segment = 0;
+    const unsigned vocab = vocab_size > 0x7fffffffu ? 0x80000000u : (unsigned) vocab_size;
+    const unsigned types = type_vocab_size > 127 ? 128u : (unsigned) type_vocab_size;
+    for (size_t i = 0; i < count; ++i) bad_id |= (unsigned) input_ids[i] >= vocab;  // a negative id wraps to a large one
+    for (size_t i = 0; i < count; ++i) bad_segment |= (unsigned) (uint8_t) segment_ids[i] >= types;
+    if (!bad_id && !bad_segment) return;
+    for (size_t i = 0; i < count; ++i) {
+        if ((unsigned) input_ids[i] >= vocab) {
+            throw std::invalid_argument("input id out of range: input_ids[" + std::to_string(i) + "] = " +
+                                        std::to_string(input_ids[i]) + ", vocab_size = " + std::to_string(vocab_size));
+        }
+    }
+    for (size_t i = 0; i < count; ++i) {
+        if ((unsigned) (uint8_t) segment_ids[i] >= types) {
+            throw std::invalid_argument("segment id out of range: segment_ids[" + std::to_string(i) + "] = " +
+                                        std::to_string((int) segment_ids[i]) + ", type_vocab_size = " +
+                                        std::to_string(type_vocab_size));
+        }
+    }
+}
+
 template <typename T>
 Bert<T>::Bert(const std::unordered_map<std::string, T *> &var, size_t max_batch_size, size_t seq_length,
               size_t vocab_size, size_t type_vocab_size, size_t hidden_size, size_t num_hidden_layers,
               size_t num_attention_heads, size_t intermediate_size, size_t num_labels)
         : max_batch_size(max_batch_size), seq_length(seq_length), hidden_size(hidden_size), num_labels(num_labels),
-          transformer(nullptr), _sequence_output(nullptr) {
+          vocab_size(vocab_size), type_vocab_size(type_vocab_size), transformer(nullptr), _sequence_output(nullptr) {
     try {
         this->stream = cuBERT::cuda_stream_create();
         this->cublas = cuBERT::blas_create();
@@ -148,6 +173,7 @@ void Bert<T>::compute(size_t batch_size, int *input_ids, int8_t *input_mask, int
         return;
     }
     const size_t M = batch_size * seq_length;
+    check_input_range(input_ids, segment_ids, M, vocab_size, type_vocab_size);
     const size_t mask_at = round_up_16(sizeof(int) * M), segments_at = round_up_16(mask_at + M);
     // The staging memory may still be being read by the previous request's copy when that request's outputs
     // were never fetched (every output method drains the stream); no event sits on a request's own path.

@@ -17,6 +17,11 @@
 
 namespace cuBERT {
 
+// Throws std::invalid_argument naming the first input id outside [0, vocab_size) or segment id outside
+// [0, type_vocab_size).  Bert<T>::compute runs it on every request before anything is enqueued.
+void check_input_range(const int *input_ids, const int8_t *segment_ids, size_t count, size_t vocab_size,
+                       size_t type_vocab_size);
+
 template <typename T>
 class Bert {
 public:
@@ -75,6 +80,7 @@ private:
     void *stream = nullptr;
 
     size_t max_batch_size, seq_length, hidden_size, num_labels;
+    size_t vocab_size, type_vocab_size;  // rows of the word and token-type tables: bounds of a request's ids
     bool has_pooler_dense, has_classifier, has_classifier_bias;
     bool classifier_head_fits = true;  // cleared when the one-launch classifier head declines this model's shape
 

@@ -1,6 +1,8 @@
 #include "Graph.h"
 
+#include <algorithm>
 #include <cstdint>
+#include <cstring>
 #include <fstream>
 #include <iostream>
 #include <stdexcept>
@@ -66,7 +68,16 @@ struct Tensor {
     int dtype = 0;
     std::vector<long long> dims;
     Reader content{nullptr, nullptr};
+    std::vector<float> float_val;      // TensorProto.float_val(5), packed or one fixed32 per tag
+    std::vector<uint16_t> half_val;    // TensorProto.half_val(13): binary16 bit patterns carried as int32
 };
+
+float fixed32_as_float(const uint8_t *p) {
+    // protobuf fixed32 is little-endian, like every host this library is built for
+    float v;
+    std::memcpy(&v, p, sizeof(v));
+    return v;
+}
 
 Tensor read_tensor(Reader r) {
     Tensor t;
@@ -76,6 +87,7 @@ Tensor read_tensor(Reader r) {
             t.dtype = (int) r.varint();
         } else if (f == 2 && w == 2) {  // TensorShapeProto
             Reader s = r.bytes();
+            t.dims.clear();  // a repeated singular message field merges; shapes are written once in practice
             uint32_t sf, sw;
             while (s.next(&sf, &sw)) {
                 if (sf == 2 && sw == 2) {  // Dim
@@ -93,12 +105,43 @@ Tensor read_tensor(Reader r) {
             }
         } else if (f == 4 && w == 2) {
             t.content = r.bytes();
+        } else if (f == 5 && w == 2) {  // packed float_val
+            Reader v = r.bytes();
+            while ((size_t) (v.end - v.p) >= 4) {
+                t.float_val.push_back(fixed32_as_float(v.p));
+                v.p += 4;
+            }
+        } else if (f == 5 && w == 5) {  // unpacked float_val
+            if ((size_t) (r.end - r.p) < 4) throw std::invalid_argument("model file invalid");
+            t.float_val.push_back(fixed32_as_float(r.p));
+            r.advance(4);
+        } else if (f == 13 && w == 2) {  // packed half_val
+            Reader v = r.bytes();
+            while (!v.done()) t.half_val.push_back((uint16_t) v.varint());
+        } else if (f == 13 && w == 0) {  // unpacked half_val
+            t.half_val.push_back((uint16_t) r.varint());
         } else {
             r.skip(w);
         }
     }
     return t;
 }
+
+// Elements a shape describes; 0 for a shape with a negative (unknown) or absurd dimension.
+size_t declared_elements(const std::vector<long long> &dims) {
+    unsigned long long n = 1;
+    for (long long d : dims) {
+        if (d < 0) return 0;
+        if (d > 0 && n > (1ull << 40) / (unsigned long long) d) return 0;
+        n *= (unsigned long long) d;
+    }
+    return (size_t) n;
+}
+
+// TensorFlow writes a constant of one element, or of many equal elements, as a short float_val / half_val
+// list instead of tensor_content; a reader repeats the last listed value up to the declared size.  Such
+// constants are scalars and splats of a few elements in a frozen BERT (epsilon, 1/sqrt(d), -10000, ...).
+constexpr size_t kMaxExpandedElements = (size_t) 1 << 24;
 
 constexpr int kDtFloat = 1, kDtHalf = 19;
 
@@ -151,6 +194,8 @@ Graph<T>::Graph(const char *filename) {
                         value = read_tensor(attr.bytes());
                         has_value = true;
                     } else {
+                        // AttrValue is a oneof over fields 1..10: the member written last is the one set
+                        if (af >= 1 && af <= 10) has_value = false;
                         attr.skip(aw);
                     }
                 }
@@ -159,36 +204,46 @@ Graph<T>::Graph(const char *filename) {
             }
         }
         if (!has_value) continue;
+        if (value.dtype != kDtFloat && value.dtype != kDtHalf) continue;
 
-        size_t len;
-        if (value.dtype == kDtFloat) len = (size_t) (value.content.end - value.content.p) / sizeof(float);
-        else if (value.dtype == kDtHalf) len = (size_t) (value.content.end - value.content.p) / sizeof(half);
-        else continue;
-
-        // a declared shape must describe the bytes that are there (a scalar has no dims)
-        unsigned long long declared = 1;
-        for (long long d : value.dims) {
-            if (d < 0 || (d > 0 && declared > (1ull << 40) / (unsigned long long) d)) {
-                throw std::invalid_argument("model file invalid: bad shape of " + name);
-            }
-            declared *= (unsigned long long) d;
-        }
-        if (declared != len) {
-            throw std::invalid_argument("model file invalid: " + name + " holds " + std::to_string(len) +
-                                        " elements, its shape says " + std::to_string(declared));
+        // The element count is what the file holds, whatever the declared shape says
+        // (reference tensorflow/Graph.cpp:50-56: len = tensor_content.len / sizeof).  The sizes of the tensors a
+        // model reads are checked where the model is built, against the shapes it needs.
+        const size_t elem = value.dtype == kDtFloat ? sizeof(float) : sizeof(half);
+        const size_t content_len = (size_t) (value.content.end - value.content.p) / elem;
+        const size_t listed = value.dtype == kDtFloat ? value.float_val.size() : value.half_val.size();
+        size_t len = content_len;
+        if (content_len == 0 && listed > 0) {
+            const size_t declared = declared_elements(value.dims);
+            len = declared >= listed && declared <= kMaxExpandedElements ? declared : listed;
         }
 
         storage.emplace_back(new T[len]);
         T *data = storage.back().get();
-        // tensor_content sits at an arbitrary byte offset of the file: copy out before converting
-        if (value.dtype == kDtFloat) {
-            std::vector<float> tmp(len);
-            std::memcpy(tmp.data(), value.content.p, len * sizeof(float));
-            T2T(tmp.data(), data, len);
-        } else {
-            std::vector<half> tmp(len);
-            std::memcpy(tmp.data(), value.content.p, len * sizeof(half));
-            T2T(tmp.data(), data, len);
+        if (content_len > 0) {
+            // tensor_content sits at an arbitrary byte offset of the file: copy out before converting
+            if (value.dtype == kDtFloat) {
+                std::vector<float> tmp(len);
+                std::memcpy(tmp.data(), value.content.p, len * sizeof(float));
+                T2T(tmp.data(), data, len);
+            } else {
+                std::vector<half> tmp(len);
+                std::memcpy(tmp.data(), value.content.p, len * sizeof(half));
+                T2T(tmp.data(), data, len);
+            }
+        } else if (len > 0) {
+            if (value.dtype == kDtFloat) {
+                std::vector<float> tmp(len, value.float_val.back());
+                std::copy(value.float_val.begin(), value.float_val.end(), tmp.begin());
+                T2T(tmp.data(), data, len);
+            } else {
+                std::vector<half> tmp(len);
+                for (size_t i = 0; i < len; ++i) {
+                    const uint16_t bits = value.half_val[i < listed ? i : listed - 1];
+                    std::memcpy(&tmp[i], &bits, sizeof(bits));
+                }
+                T2T(tmp.data(), data, len);
+            }
         }
         var[name] = data;  // a repeated name keeps its last tensor
         shape[name] = value.dims;

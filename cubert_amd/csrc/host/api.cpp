@@ -169,6 +169,18 @@ void transformer_run(const char *prefix, int n, const char *const *names, const 
     cuBERT::cuda_stream_destroy(stream);
 }
 
+template <typename T>
+const void *graph_var(const cuBERT::Graph<T> *g, const char *name, size_t *elements, long long *dims, int max_dims,
+                      int *n_dims) {
+    auto it = g->var.find(name);
+    if (it == g->var.end()) return nullptr;
+    if (elements != nullptr) *elements = g->size.at(name);
+    const std::vector<long long> &shape = g->shape.at(name);
+    if (n_dims != nullptr) *n_dims = (int) shape.size();
+    for (int i = 0; dims != nullptr && i < max_dims && i < (int) shape.size(); ++i) dims[i] = shape[i];
+    return it->second;
+}
+
 }  // namespace
 
 extern "C" {
@@ -402,6 +414,56 @@ int cubert_bert_destroy(void *bert, int dtype) {
     return guarded([&] {
         if (dtype == 0) delete (cuBERT::Bert<float> *) bert;
         else delete (cuBERT::Bert<half> *) bert;
+    });
+}
+
+int cubert_check_input_range(const int *input_ids, const int8_t *segment_ids, size_t count, size_t vocab_size,
+                             size_t type_vocab_size) {
+    return guarded([&] {
+        if (count > 0 && (input_ids == nullptr || segment_ids == nullptr)) throw std::invalid_argument("null argument");
+        cuBERT::check_input_range(input_ids, segment_ids, count, vocab_size, type_vocab_size);
+    });
+}
+
+int cubert_graph_open(const char *model_file, int dtype, void **graph) {
+    return guarded([&] {
+        if (graph == nullptr || model_file == nullptr) throw std::invalid_argument("null argument");
+        *graph = dtype == 0 ? (void *) new cuBERT::Graph<float>(model_file) : (void *) new cuBERT::Graph<half>(model_file);
+    });
+}
+
+long long cubert_graph_count(void *graph, int dtype) {
+    if (graph == nullptr) return -1;
+    return dtype == 0 ? (long long) ((cuBERT::Graph<float> *) graph)->var.size()
+                      : (long long) ((cuBERT::Graph<half> *) graph)->var.size();
+}
+
+const void *cubert_graph_var(void *graph, int dtype, const char *name, size_t *elements, long long *dims,
+                             int max_dims, int *n_dims) {
+    if (graph == nullptr || name == nullptr) return nullptr;
+    return dtype == 0 ? graph_var((const cuBERT::Graph<float> *) graph, name, elements, dims, max_dims, n_dims)
+                      : graph_var((const cuBERT::Graph<half> *) graph, name, elements, dims, max_dims, n_dims);
+}
+
+int cubert_graph_sizes(void *graph, int dtype, size_t sizes[5]) {
+    return guarded([&] {
+        if (graph == nullptr || sizes == nullptr) throw std::invalid_argument("null argument");
+        auto fill = [&](auto *g) {
+            sizes[0] = g->vocab_size;
+            sizes[1] = g->type_vocab_size;
+            sizes[2] = g->hidden_size;
+            sizes[3] = g->intermediate_size;
+            sizes[4] = g->num_labels;
+        };
+        if (dtype == 0) fill((cuBERT::Graph<float> *) graph);
+        else fill((cuBERT::Graph<half> *) graph);
+    });
+}
+
+int cubert_graph_close(void *graph, int dtype) {
+    return guarded([&] {
+        if (dtype == 0) delete (cuBERT::Graph<float> *) graph;
+        else delete (cuBERT::Graph<half> *) graph;
     });
 }
 

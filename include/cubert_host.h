@@ -50,10 +50,27 @@ int cubert_try_compute(void *model, int batch_size, int *input_ids, int8_t *inpu
 /* replaces: cuBERT_compute_m, reference src/cuBERT.cpp:69-90 */
 int cubert_try_compute_m(void *model, int batch_size, int *input_ids, int8_t *input_mask, int8_t *segment_ids,
                          cuBERT_Output *output, int compute_type, int output_to_float);
+/* The range check cuBERT_compute applies to a request before anything is enqueued: every input id in
+ * [0, vocab_size), every segment id in [0, type_vocab_size); CUBERT_E_INVALID_ARGUMENT and a message naming the
+ * first offender otherwise.  (The reference indexes its tables unchecked, src/cuBERT/op/Embedding.cpp:16-19.) */
+int cubert_check_input_range(const int *input_ids, const int8_t *segment_ids, size_t count, size_t vocab_size,
+                             size_t type_vocab_size);
 /* replaces: cuBERT_close, reference src/cuBERT.cpp:92-102 */
 int cubert_try_close(void *model, int compute_type);
 /* Shape facts of an opened model (hidden size, labels, seq_length) for sizing output arrays. */
 int cubert_model_info(void *model, int compute_type, int *hidden_size, int *num_labels, int *seq_length);
+/* replaces: Graph<T>::Graph(filename) and the public members of Graph<T>, reference
+ * src/cuBERT/tensorflow/Graph.h:10-23, Graph.cpp:13-91: the float and binary16 constants of a frozen GraphDef
+ * converted to dtype (0 float, 1 binary16), by node name.  CPU only.  cubert_graph_var gives the host pointer the
+ * graph owns (NULL for an unknown name), the number of elements it holds and, when dims != NULL, up to max_dims
+ * dimensions of the declared shape (*n_dims receives the rank).  cubert_graph_sizes gives vocab_size,
+ * type_vocab_size, hidden_size, intermediate_size and num_labels in that order. */
+int cubert_graph_open(const char *model_file, int dtype, void **graph);
+long long cubert_graph_count(void *graph, int dtype);
+const void *cubert_graph_var(void *graph, int dtype, const char *name, size_t *elements, long long *dims,
+                             int max_dims, int *n_dims);
+int cubert_graph_sizes(void *graph, int dtype, size_t sizes[5]);
+int cubert_graph_close(void *graph, int dtype);
 /* replaces: cuBERT_open_tokenizer, reference src/cuBERT.cpp:104-106 */
 int cubert_try_open_tokenizer(const char *vocab_file, int do_lower_case, void **tokenizer);
 /* replaces: cuBERT_tokenize_compute / cuBERT_tokenize_compute_m, reference src/cuBERT.cpp:216-280 */

@@ -104,6 +104,77 @@ def test_graphdef_wire_format_matches_protobuf_library(tmp_path):
     assert np.array_equal(np.frombuffer(tensor[4], np.float32), np.arange(6, dtype=np.float32))
 
 
+from util import tf_style_fixture
+
+
+@pytest.mark.parametrize("compute_type", [0, 1])
+def test_loader_reads_a_graphdef_written_the_way_tensorflow_writes_one(compute_type):
+    """Scalars and splats in float_val / half_val (packed and unpacked), a weight stored as DT_HALF, non-Const
+    nodes, a fixed32 attr, int32 Consts, versions and a function library, a repeated name: every float / half
+    constant arrives bit-exact (after conversion to the model's type), nothing else does, nothing throws."""
+    import cubert_amd
+    path, expected, absent = tf_style_fixture()
+    g = cubert_amd.Graph(path, compute_type)
+    assert (g.vocab_size, g.type_vocab_size, g.hidden_size, g.intermediate_size, g.num_labels) == (37, 2, 16, 32, 3)
+    assert len(g) == len(expected)
+    for name, want in expected.items():
+        got = g.var(name)
+        assert got is not None, name
+        data, shape = got
+        want = want.astype(np.float32 if compute_type == 0 else np.float16)
+        assert data.shape == (want.size,), (name, data.shape, want.shape)
+        assert np.array_equal(data.view(np.uint32 if compute_type == 0 else np.uint16),
+                              want.reshape(-1).view(np.uint32 if compute_type == 0 else np.uint16)), name
+    assert g.var("bert/embeddings/word_embeddings")[1] == (37, 16)
+    assert g.var("bert/embeddings/LayerNorm/batchnorm/add/y")[1] == ()
+    # the function library's Const of the same name did not replace the weight
+    assert not np.any(g.var("bert/embeddings/LayerNorm/beta")[0] == 99)
+    for name in absent:
+        assert g.var(name) is None, name
+    g.close()
+
+
+def test_loader_keeps_what_the_file_holds_when_the_declared_shape_disagrees(tmp_path):
+    """The element count of a constant is the length of its tensor_content, whatever its shape says (reference
+    tensorflow/Graph.cpp:50-56); a model whose tensors do not fit is refused where it is built, by name."""
+    import cubert_amd
+    from cubert_amd.graphdef import _bytes_field, _field, _varint
+    content = np.arange(5, dtype=np.float32).tobytes()
+    shape = _bytes_field(2, _field(1, 0, _varint(2))) + _bytes_field(2, _field(1, 0, _varint(3)))   # says [2, 3]
+    tensor = _field(1, 0, _varint(1)) + _bytes_field(2, shape) + _bytes_field(4, content)
+    # AttrValue with the tensor first and another member of the oneof after it: the later member is the one set
+    overwritten = _bytes_field(8, tensor) + _field(3, 0, _varint(7))
+    nodes = b""
+    for name, attr in (("odd/shape", _bytes_field(8, tensor)), ("odd/oneof", overwritten)):
+        entry = _bytes_field(1, b"value") + _bytes_field(2, attr)
+        nodes += _bytes_field(1, _bytes_field(1, name.encode()) + _bytes_field(2, b"Const") + _bytes_field(5, entry))
+    path = tmp_path / "odd.pb"
+    path.write_bytes(nodes)
+    g = cubert_amd.Graph(str(path))
+    data, shape = g.var("odd/shape")
+    assert shape == (2, 3) and np.array_equal(data, np.arange(5, dtype=np.float32))
+    assert g.var("odd/oneof") is None and len(g) == 1
+    g.close()
+    # truncated in the middle of a node: an error, not a crash
+    (tmp_path / "cut.pb").write_bytes(nodes[:len(nodes) - 9])
+    with pytest.raises(ValueError, match="model file invalid"):
+        cubert_amd.Graph(str(tmp_path / "cut.pb"))
+    with pytest.raises(ValueError, match="model file not found"):
+        cubert_amd.Graph(str(tmp_path / "missing.pb"))
+
+
+def test_open_accepts_the_tensorflow_style_file_up_to_the_device_check():
+    """cuBERT_open on the fixture: the loader and the size checks pass (seq_length 8 of 12 positions), and without a
+    GPU the call ends at the device count like the reference's (BertM.cpp:20-22)."""
+    import cubert_amd
+    path, _, _ = tf_style_fixture()
+    if cubert_amd.get_gpu_count() == 0:
+        with pytest.raises(ValueError, match="No GPU device detected"):
+            cubert_amd.Model(path, 4, 8, 2, 2)
+    with pytest.raises(ValueError, match="position_embeddings holds 192 elements, the model needs 256"):
+        cubert_amd.Model(path, 4, 16, 2, 2)
+
+
 def test_generators_are_deterministic_and_follow_the_configs():
     from cubert_amd.testing import CONFIGS, config_inputs, random_bert_weights
     small = dict(vocab=50, hidden=16, layers=2, heads=2, intermediate=32, max_position=8, type_vocab=2)
@@ -158,6 +229,32 @@ def test_open_rejects_files_whose_tensors_do_not_fit_the_model(tmp_path):
             open_(w)
     else:
         open_(w)
+
+
+def test_input_range_check():
+    """What Bert<T>::compute checks before it enqueues anything: ids in [0, vocab), segment ids in [0, types)."""
+    from cubert_amd._lib import lib
+    L = lib()
+    ids = np.array([0, 5, 20, 99, 3], np.int32)
+    seg = np.array([0, 1, 0, 1, 1], np.int8)
+
+    def check(i, s, vocab, types):
+        rc = L.cubert_check_input_range(i.ctypes.data, s.ctypes.data, i.size, vocab, types)
+        return rc, L.cubert_last_error().decode()
+
+    assert check(ids, seg, 100, 2) == (0, "")
+    assert check(ids[:0], seg[:0], 100, 2) == (0, "")
+    assert check(ids, seg, 99, 2) == (1, "input id out of range: input_ids[3] = 99, vocab_size = 99")
+    neg = ids.copy()
+    neg[1] = -7
+    assert check(neg, seg, 100, 2) == (1, "input id out of range: input_ids[1] = -7, vocab_size = 100")
+    assert check(ids, seg, 100, 1) == (1, "segment id out of range: segment_ids[1] = 1, type_vocab_size = 1")
+    bad = seg.copy()
+    bad[4] = -1
+    assert check(ids, bad, 100, 2) == (1, "segment id out of range: segment_ids[4] = -1, type_vocab_size = 2")
+    big = np.arange(1 << 15, dtype=np.int32)
+    assert check(big, np.zeros(big.size, np.int8), 1 << 15, 2)[0] == 0
+    assert check(big, np.zeros(big.size, np.int8), (1 << 15) - 1, 2)[0] == 1
 
 
 def test_bench_refuses_more_than_one_gpu():
