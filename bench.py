@@ -5,12 +5,20 @@
 
 A step is one forward pass of the workload (default C1: BERT-base fp32, batch 128, seq_len 32,
 the configuration the headline metric is quoted on) on inputs already resident in device memory.
-Prints ONE JSON line: sequences/s over the K timed steps, the roofline of the dominant fused
-kernel (bias+GELU) measured with HIP events around its launches inside the timed steps, and the
-CPU oracle timed on this host's cores on a bounded sample of the same workload.
+Prints ONE JSON line:
+  value / ms_per_step   sequences/s over the K timed device-resident steps
+  roofline              the dominant fused kernel (bias+GELU), HIP events around its launches inside the timed steps
+  kernels               every kernel kind of the forward pass: average launch time, GB/s, fraction of the HBM peak
+  clean_roofline        the same table at C3 (BERT-base fp16, batch 64, seq_len 512), whose tensors do not fit the
+                        256 MB Infinity Cache: the workload where a fraction of the HBM peak is an HBM statement
+  host_path             the reference benchmark client's protocol (benchmark/benchmark_cu.cpp:68-78): host arrays in,
+                        POOLED_OUTPUT out, 10 warm-up calls, then timed calls (PCIe-inclusive)
+  cpu_baseline          the CPU oracle on this host's cores on a bounded sample of the same workload, with the
+                        thread counts the libraries report and the time per part of a pass
 """
 import argparse
 import faulthandler
+import hashlib
 import json
 import os
 import sys
@@ -25,7 +33,17 @@ HBM_PEAK_GBS = 8000.0
 
 # Bytes per launch that crossed the L2 <-> memory boundary, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script scaled by a plain copy of known size (method and table: profiles/traffic_pmc.md).  Hardware counters
-# need the profiler, so these are recorded values, not measured by a plain run.
+# need the profiler, so these are recorded values, not measured by a plain run: each is tied to the SHA-256 of the
+# kernel source it was measured on and is reported only while that file is unchanged.
+TRAFFIC_PROFILE = "profiles/traffic_pmc.md"
+TRAFFIC_SOURCE = {  # kernel kind -> (source file under cubert_amd/csrc/kernels, first 16 hex digits of its SHA-256)
+    "bias_gelu": ("elementwise.hip", "59dcc33f61344079"),
+    "bias_tanh": ("elementwise.hip", "59dcc33f61344079"),
+    "bias_res_ln": ("layernorm.hip", "3fc1f92646a53b40"),
+    "embed_ln": ("layernorm.hip", "3fc1f92646a53b40"),
+    "mask_scale_softmax": ("softmax.hip", "90a529eac55169fa"),
+    "attention_fused": ("attention.hip", "ca1212b0708528de"),
+}
 MEASURED_TRAFFIC = {
     "C1": {
         "attention_fused": 50675000,
@@ -35,7 +53,7 @@ MEASURED_TRAFFIC = {
         "bias_gelu": 100321862
     },
     "C3": {
-        "attention_fused": 200310000,
+        "attention_fused": 124900000,
         "embed_ln": 99683567,
         "mask_scale_softmax": 801872210,
         "bias_res_ln": 150175758,
@@ -50,6 +68,25 @@ MEASURED_TRAFFIC = {
         "bias_tanh": 1110678
     }
 }
+
+
+def recorded_traffic(workload, kind):
+    """(bytes per launch or None, where the figure comes from / why it is withheld)."""
+    value = MEASURED_TRAFFIC.get(workload, {}).get(kind)
+    if value is None or kind not in TRAFFIC_SOURCE:
+        return None, "no hardware-counter run recorded for this kernel and workload"
+    name, digest = TRAFFIC_SOURCE[kind]
+    path = os.path.join(ROOT, "cubert_amd", "csrc", "kernels", name)
+    try:
+        with open(path, "rb") as f:
+            now = hashlib.sha256(f.read()).hexdigest()[:16]
+    except OSError:
+        return None, "kernel source %s not found" % name
+    if now != digest:
+        return None, "%s changed since the counter run recorded in %s (then %s, now %s)" % (name, TRAFFIC_PROFILE,
+                                                                                           digest, now)
+    return value, "recorded, not measured by this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, %s; %s unchanged " \
+                  "since (sha256 %s)" % (TRAFFIC_PROFILE, name, digest)
 
 
 def two_term_dense():
@@ -153,6 +190,84 @@ def standalone_kernel(kind, cfg, mask, alg_bytes, reps=20):
                     "another kernel (%s)" % ("attention_fused" if kind == "mask_scale_softmax" else "the few-token Dense")}
 
 
+def kernel_table(bert, cfg, mask, alg, batch, passes):
+    """Every kernel kind of `passes` forward passes with an event pair around each launch:
+    {kind: average microseconds, launches, and for the fused kernels GB/s and fraction of the HBM peak}."""
+    table = {}
+    bert.profile([k for k in bert.KINDS])
+    for _ in range(passes):
+        bert.compute_resident(batch)
+    for k, (ms, n) in bert.profile_read().items():
+        us = ms * 1e3 / n
+        table[k] = {"avg_us": round(us, 2), "launches": n}
+        if k in alg:
+            table[k]["GB/s"] = round(alg[k] / (us * 1e-6) / 1e9, 1)
+            table[k]["frac_hbm_peak"] = round(alg[k] / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
+    bert.profile([])
+    # the forward pass runs the attention core as one kernel where the shape allows and then never launches the
+    # mask + scale + softmax kernel, and at <= 32 tokens bias + GELU runs inside the few-token Dense kernel: those are
+    # timed by themselves at the workload's shape
+    for kind in ("mask_scale_softmax", "bias_gelu"):
+        if kind not in table:
+            table[kind] = standalone_kernel(kind, cfg, mask, alg[kind])
+    return table
+
+
+def cpu_baseline(workload, cfg, w, ids, mask, seg):
+    """The oracle (a port of the reference's CPU path) on this host's cores: a bounded sample of the workload at the
+    default thread count and at 4 threads (the reference's CI setting, .travis.yml:25), each with the thread counts
+    the libraries report for themselves and the seconds per part of a pass."""
+    import ctypes
+    import oracle
+    m = cfg["model"]
+    S = cfg["seq_length"]
+    half = cfg["dtype"] == "f16"
+    default_threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    oracle.lib()
+    try:
+        gomp = ctypes.CDLL("libgomp.so.1")
+    except OSError:
+        gomp = None
+    wf = {k: oracle.round_to_half(v) for k, v in w.items()} if half else w
+    vars_obj = oracle.Vars(wf)
+    n = min(cfg["batch"], 128)  # bounded sample: at most 128 sequences of the workload per pass
+
+    def leg(threads, max_passes, budget_s):
+        oracle.set_blas_threads(threads)
+        if gomp is not None:
+            gomp.omp_set_num_threads(threads)
+        oracle.bert_forward(wf, ids[:n], mask[:n], seg[:n], m["layers"], m["heads"], vars_obj=vars_obj)  # warm-up
+        oracle.profile_reset()
+        times = []
+        start = time.perf_counter()
+        while len(times) < max_passes and time.perf_counter() - start < budget_s:
+            t = time.perf_counter()
+            oracle.bert_forward(wf, ids[:n], mask[:n], seg[:n], m["layers"], m["heads"], vars_obj=vars_obj)
+            times.append(time.perf_counter() - t)
+        parts = {k: round(v / len(times) * 1e3, 1) for k, v in oracle.profile_read().items()}
+        return {"value": round(n / float(np.mean(times)), 2), "passes": len(times),
+                "ms_per_pass": round(float(np.mean(times)) * 1e3, 1), "ms_per_pass_by_part": parts,
+                "threads": oracle.threads_in_use()}
+
+    main_leg = leg(default_threads, 3, 20)
+    four = leg(4, 2, 10) if default_threads > 4 else None
+    oracle.set_blas_threads(default_threads)
+    if gomp is not None:
+        gomp.omp_set_num_threads(default_threads)
+    dense = main_leg["ms_per_pass_by_part"]["dense_gemm"]
+    M, H, I = n * S, m["hidden"], m["intermediate"]
+    dense_flop = 2.0 * M * (4 * H * H + 2 * H * I) * m["layers"]
+    return {"value": main_leg["value"], "unit": "sequences/s", "cores": default_threads, "kind": "port",
+            "sample": "%d pass(es) of %d sequences of %s (seq_len %d), fp32, mean %.1f ms/pass" %
+                      (main_leg["passes"], n, workload, S, main_leg["ms_per_pass"]),
+            "blas": os.path.basename(oracle.blas_name()),
+            "label": "restatement of the reference's CPU path on OpenBLAS (attention batches as an OpenMP loop around "
+                     "single-threaded sgemm calls, the way cblas_sgemm_batch spreads a group)",
+            "threads": main_leg["threads"], "ms_per_pass_by_part": main_leg["ms_per_pass_by_part"],
+            "dense_gemm_GFLOPs": round(dense_flop / (dense * 1e-3) / 1e9, 1) if dense > 0 else None,
+            "value_at_4_threads": four["value"] if four else None, "at_4_threads": four}
+
+
 def main():
     faulthandler.enable()  # a crash inside the native library prints the Python stack
     ap = argparse.ArgumentParser()
@@ -161,7 +276,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="C1")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--all-kernels", action="store_true", help="time every kernel kind in an extra untimed pass")
+    ap.add_argument("--all-kernels", action="store_true",
+                    help="kept for old command lines: the per-kernel table is always part of the line now")
+    ap.add_argument("--no-clean-leg", action="store_true",
+                    help="skip the extra leg that times every kernel at C3 (fp16, batch 64, seq_len 512), the workload "
+                         "whose tensors do not fit the Infinity Cache (run by default when the workload is C1)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="instead of the model: 10 launches of a plain row copy of known size (100 MB read, 100 MB "
                          "written), the yardstick for hardware traffic counters")
@@ -231,7 +350,8 @@ def main():
     value = B / (ms_per_step * 1e-3)
 
     alg = algorithmic_bytes(cfg)
-    traffic = None if two_term_dense() else MEASURED_TRAFFIC.get(args.workload, {}).get(dominant)
+    traffic, traffic_source = (None, "no counter run recorded for the two-term form") if two_term_dense() \
+        else recorded_traffic(args.workload, dominant)
     if dominant in prof:
         total_ms, launches = prof[dominant]
         avg_us = total_ms * 1e3 / launches
@@ -240,28 +360,11 @@ def main():
         avg_us, launches = alone["avg_us"], alone["launches"]
     achieved = alg[dominant] / (avg_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
                 "algorithmic_bytes_per_launch": alg[dominant], "avg_launch_us": round(avg_us, 2), "launches": launches}
 
-    # ---- every kernel kind, in an extra untimed pass (reported, not part of `value`)
-    kernels = {}
-    if args.all_kernels:
-        bert.profile([k for k in bert.KINDS])
-        for _ in range(max(5, args.steps // 5)):
-            bert.compute_resident(B)
-        for k, (ms, n) in bert.profile_read().items():
-            us = ms * 1e3 / n
-            kernels[k] = {"avg_us": round(us, 2), "launches": n}
-            if k in alg:
-                kernels[k]["GB/s"] = round(alg[k] / (us * 1e-6) / 1e9, 1)
-                kernels[k]["frac_hbm_peak"] = round(alg[k] / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
-        bert.profile([])
-        if "mask_scale_softmax" not in kernels:
-            # the forward pass runs the attention core as one kernel where the shape allows and then never launches the
-            # mask + scale + softmax kernel.  Time it by itself on a score tensor of the workload's shape.
-            kernels["mask_scale_softmax"] = standalone_kernel("mask_scale_softmax", cfg, mask, alg["mask_scale_softmax"])
-        if "bias_gelu" not in kernels:
-            kernels["bias_gelu"] = standalone_kernel("bias_gelu", cfg, mask, alg["bias_gelu"])
+    # ---- every kernel kind, in extra untimed passes (reported, not part of `value`)
+    kernels = kernel_table(bert, cfg, mask, alg, B, max(5, args.steps // 5))
 
     # ---- the public path: host arrays in, host array out (PCIe-inclusive), and p50 latency at batch 1
     host_path, p50_b1 = None, None
@@ -286,6 +389,32 @@ def main():
                 lat1.append((time.perf_counter() - t) * 1e3)
         p50_b1 = round(float(np.median(lat1)), 3)
     bert.close()
+
+    # ---- every kernel at C3, where the tensors do not fit the Infinity Cache (same weights: both are BERT-base)
+    clean = None
+    if args.workload == "C1" and not args.device_only and not args.no_clean_leg and not two_term_dense():
+        c3 = CONFIGS["C3"]
+        ids3, mask3, seg3 = config_inputs("C3", seed=0)
+        big = cubert_amd.Bert(w, c3["batch"], c3["seq_length"], m["layers"], m["heads"], 1)
+        big.compute(ids3, mask3, seg3)
+        big.synchronize()
+        for _ in range(3):
+            big.compute_resident(c3["batch"])
+        big.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            big.compute_resident(c3["batch"])
+        big.synchronize()
+        ms3 = (time.perf_counter() - t0) * 1e3 / 10
+        alg3 = algorithmic_bytes(c3)
+        table3 = kernel_table(big, c3, mask3, alg3, c3["batch"], 5)
+        big.close()
+        for k, row in table3.items():
+            row["traffic"], _ = recorded_traffic("C3", k)
+        clean = {"workload": "C3: BERT-base f16 batch %d seq_len %d, valid length min(512, 16 + Exp(96)), inputs "
+                             "resident in HBM" % (c3["batch"], c3["seq_length"]),
+                 "ms_per_step": round(ms3, 4), "sequences_per_s": round(c3["batch"] / (ms3 * 1e-3), 1), "steps": 10,
+                 "kernels": table3}
 
     # ---- the same steps with the opt-in two-term fp16 Dense form of fp32 models (reported beside `value`, never as it)
     two_term = None
@@ -347,43 +476,7 @@ def main():
     # ---- CPU baseline: the oracle (a port of the reference's CPU path) on this host's cores
     cpu = None
     if not args.no_cpu and not args.device_only:
-        import oracle
-        threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-        oracle.lib()
-        oracle.set_blas_threads(threads)
-        wf = {k: oracle.round_to_half(v) for k, v in w.items()} if half else w
-        vars_obj = oracle.Vars(wf)
-        # bounded sample: at most 128 sequences of the workload per pass, 1 warm-up + up to 3 timed passes or ~20 s
-        n = min(B, 128)
-        oracle.bert_forward(wf, ids[:n], mask[:n], seg[:n], m["layers"], m["heads"], vars_obj=vars_obj)
-        times = []
-        start = time.perf_counter()
-        while len(times) < 3 and time.perf_counter() - start < 20:
-            t = time.perf_counter()
-            oracle.bert_forward(wf, ids[:n], mask[:n], seg[:n], m["layers"], m["heads"], vars_obj=vars_obj)
-            times.append(time.perf_counter() - t)
-        # the same at 4 threads, the thread count of the reference's CI run of its CPU path
-        four = None
-        if threads > 4:
-            import ctypes
-            oracle.set_blas_threads(4)
-            try:
-                ctypes.CDLL("libgomp.so.1").omp_set_num_threads(4)
-            except OSError:
-                pass
-            oracle.bert_forward(wf, ids[:n], mask[:n], seg[:n], m["layers"], m["heads"], vars_obj=vars_obj)
-            t4 = []
-            start = time.perf_counter()
-            while len(t4) < 2 and time.perf_counter() - start < 10:
-                t = time.perf_counter()
-                oracle.bert_forward(wf, ids[:n], mask[:n], seg[:n], m["layers"], m["heads"], vars_obj=vars_obj)
-                t4.append(time.perf_counter() - t)
-            four = round(n / float(np.mean(t4)), 2)
-        cpu = {"value": round(n / float(np.mean(times)), 2), "unit": "sequences/s", "cores": threads, "kind": "port",
-               "value_at_4_threads": four,
-               "sample": "%d pass(es) of %d sequences of %s (seq_len %d), fp32, mean %.1f ms/pass" %
-                         (len(times), n, args.workload, S, float(np.mean(times)) * 1e3),
-               "blas": os.path.basename(oracle.blas_name())}
+        cpu = cpu_baseline(args.workload, cfg, w, ids, mask, seg)
 
     line = {
         "metric": "sequences/s, BERT forward pass (%s)" % args.workload,
@@ -391,7 +484,9 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": cfg["dtype"], "data": "synthetic",
         "config": {"workload": "%s: %s %s batch %d seq_len %d, random-init N(0,0.02) weights, inputs resident in HBM" %
-                               (args.workload, "BERT-large" if m["hidden"] == 1024 else "BERT-base", cfg["dtype"], B, S)},
+                               (args.workload, "BERT-large" if m["hidden"] == 1024 else "BERT-base", cfg["dtype"], B, S),
+                   "value_is": "device-resident forward passes; the host-arrays-in / host-array-out protocol of the "
+                               "reference's benchmark client is `host_path`"},
         "roofline": roofline, "cpu_baseline": cpu,
         "p50_ms_batch1_host_path": p50_b1, "host_path": host_path,
     }
@@ -401,8 +496,11 @@ def main():
         line["two_term_fp16_dense"] = two_term
     if concurrent is not None:
         line["concurrent_instances"] = concurrent
-    if kernels:
-        line["kernels"] = kernels
+    for k, row in kernels.items():
+        row["traffic"], _ = recorded_traffic(args.workload, k)
+    line["kernels"] = kernels
+    if clean is not None:
+        line["clean_roofline"] = clean
     print(json.dumps(line))
 
 

@@ -105,6 +105,42 @@ def set_blas_threads(n):
     return True
 
 
+def set_batch_parallel(on):
+    """Batched attention GEMMs as an OpenMP loop around single-threaded BLAS calls (default) or one multi-threaded
+    call per problem."""
+    lib().oracle_set_batch_parallel(int(bool(on)))
+
+
+PROFILE_PARTS = ("dense_gemm", "attention_batch_gemm", "row_kernels", "other")
+
+
+def profile_reset():
+    lib().oracle_profile_reset()
+
+
+def profile_read():
+    """Seconds per part of the forward passes since the last reset."""
+    out = (ctypes.c_double * len(PROFILE_PARTS))()
+    lib().oracle_profile_read(out)
+    return dict(zip(PROFILE_PARTS, (float(v) for v in out)))
+
+
+def threads_in_use():
+    """What the host and the libraries report about themselves: logical CPUs, CPUs this process may run on, the
+    OpenMP team size of the oracle's loops and the thread count of the loaded BLAS."""
+    info = {"nproc": os.cpu_count(), "OMP_NUM_THREADS": os.environ.get("OMP_NUM_THREADS"),
+            "blas_threads": int(lib().oracle_blas_threads())}
+    try:
+        info["sched_affinity"] = len(os.sched_getaffinity(0))
+    except AttributeError:
+        info["sched_affinity"] = None
+    try:
+        info["omp_max_threads"] = int(ctypes.CDLL("libgomp.so.1").omp_get_max_threads())
+    except OSError:
+        info["omp_max_threads"] = None
+    return info
+
+
 class Vars(object):
     """Named fp32 weights in the form the C oracle takes them (names + pointers)."""
 

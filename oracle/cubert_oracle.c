@@ -9,6 +9,7 @@
 #include <dlfcn.h>
 #include <float.h>
 #include <math.h>
+#include <omp.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -22,6 +23,22 @@ typedef void (*cblas_sgemm_fn)(int order, int transA, int transB, int M, int N, 
 static cblas_sgemm_fn g_sgemm = NULL;
 static void *g_blas_handle = NULL;
 static char g_blas_name[512] = "builtin triple loop";
+static void (*g_blas_set_threads)(int) = NULL; /* the loaded BLAS's own thread-count calls, when it has them */
+static int (*g_blas_get_threads)(void) = NULL;
+static int g_batch_parallel = 1;
+
+/* Wall-clock seconds per part of a forward pass, for the CPU baseline's breakdown (not used by any test). */
+static double g_seconds[ORACLE_PROFILE_PARTS];
+#define TIMED(part, call)                      \
+    do {                                       \
+        double t0_ = omp_get_wtime();          \
+        call;                                  \
+        g_seconds[part] += omp_get_wtime() - t0_; \
+    } while (0)
+
+void oracle_profile_reset(void) { memset(g_seconds, 0, sizeof g_seconds); }
+
+void oracle_profile_read(double seconds[ORACLE_PROFILE_PARTS]) { memcpy(seconds, g_seconds, sizeof g_seconds); }
 
 int oracle_use_cblas(const char *path, const char *sym) {
     void *h = dlopen(path, RTLD_NOW | RTLD_LOCAL);
@@ -33,12 +50,27 @@ int oracle_use_cblas(const char *path, const char *sym) {
     }
     g_blas_handle = h;
     g_sgemm = (cblas_sgemm_fn) f;
+    g_blas_set_threads = NULL;
+    g_blas_get_threads = NULL;
+    {
+        const char *setters[] = {"scipy_openblas_set_num_threads", "openblas_set_num_threads", "MKL_Set_Num_Threads"};
+        const char *getters[] = {"scipy_openblas_get_num_threads", "openblas_get_num_threads", "MKL_Get_Max_Threads"};
+        for (int i = 0; i < 3 && !g_blas_set_threads; ++i) {
+            void *set = dlsym(h, setters[i]), *get = dlsym(h, getters[i]);
+            if (set && get) {
+                g_blas_set_threads = (void (*)(int)) set;
+                g_blas_get_threads = (int (*)(void)) get;
+            }
+        }
+    }
     snprintf(g_blas_name, sizeof g_blas_name, "%s:%s", path, sym);
     return 0;
 }
 
 void oracle_use_builtin_gemm(void) {
     g_sgemm = NULL;
+    g_blas_set_threads = NULL;
+    g_blas_get_threads = NULL;
     snprintf(g_blas_name, sizeof g_blas_name, "builtin triple loop");
 }
 
@@ -70,6 +102,32 @@ void oracle_sgemm(int transA, int transB, int M, int N, int K, float alpha, cons
                 lda, B, ldb, beta, C, ldc);
     } else {
         builtin_sgemm(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);
+    }
+}
+
+void oracle_set_batch_parallel(int on) { g_batch_parallel = on != 0; }
+
+int oracle_blas_threads(void) { return g_blas_get_threads ? g_blas_get_threads() : 0; }
+
+/* reference: common.cpp:260-298 (blas_gemm_batch<float>, HAVE_MKL branch): one cblas_sgemm_batch group of
+ * `count` independent problems of one shape.  MKL spreads the problems of a group over its threads; here
+ * the problems are an OpenMP loop around single-threaded sgemm calls when the loaded BLAS lets its thread count
+ * be set (oracle_set_batch_parallel(0): one multi-threaded sgemm per problem, in order).  Either way every
+ * problem is the same sgemm on the same operands. */
+void oracle_sgemm_batch(int transA, int transB, int M, int N, int K, float alpha, const float **A, int lda,
+                        const float **B, int ldb, float beta, float **C, int ldc, int count) {
+    if (g_sgemm && g_batch_parallel && g_blas_set_threads && count > 1 && omp_get_max_threads() > 1) {
+        int before = g_blas_get_threads();
+        g_blas_set_threads(1);
+#pragma omp parallel for schedule(static)
+        for (int i = 0; i < count; ++i) {
+            g_sgemm(102, transA ? 112 : 111, transB ? 112 : 111, M, N, K, alpha, A[i], lda, B[i], ldb, beta, C[i], ldc);
+        }
+        g_blas_set_threads(before);
+        return;
+    }
+    for (int i = 0; i < count; ++i) {
+        oracle_sgemm(transA, transB, M, N, K, alpha, A[i], lda, B[i], ldb, beta, C[i], ldc);
     }
 }
 
@@ -200,33 +258,47 @@ void oracle_attention_mask(int batch, int seq_length, int heads, const int8_t *m
 }
 
 /* reference: op_att/BatchMatMul.cpp:31-38 (per-(b,h) base pointers) and
- * :57-68 (gemm T,N m=n=S k=d, lda=ldb=H, ldc=S*A). */
+ * :57-68 (gemm_batch T,N m=n=S k=d, lda=ldb=H, ldc=S*A). */
 void oracle_att_q_k(int batch, int seq_length, int heads, int size_per_head, const float *query,
                     const float *key, float *scores, float alpha, float beta) {
-    int S = seq_length, A = heads, d = size_per_head;
+    int S = seq_length, A = heads, d = size_per_head, count = batch * heads;
+    const float **q = (const float **) malloc(sizeof(float *) * (size_t) count);
+    const float **k = (const float **) malloc(sizeof(float *) * (size_t) count);
+    float **out = (float **) malloc(sizeof(float *) * (size_t) count);
     for (int b = 0; b < batch; ++b) {
         for (int h = 0; h < A; ++h) {
             size_t idx = (size_t) b * S * d * A + (size_t) d * h;
-            float *out = scores + (size_t) b * S * S * A + (size_t) S * h;
-            oracle_sgemm(1, 0, S, S, d, alpha, key + idx, d * A, query + idx, d * A, beta, out,
-                         S * A);
+            q[b * A + h] = query + idx;
+            k[b * A + h] = key + idx;
+            out[b * A + h] = scores + (size_t) b * S * S * A + (size_t) S * h;
         }
     }
+    oracle_sgemm_batch(1, 0, S, S, d, alpha, k, d * A, q, d * A, beta, out, S * A, count);
+    free(out);
+    free(k);
+    free(q);
 }
 
 /* reference: op_att/BatchMatMul.cpp:103-110 and :129-140
- * (gemm N,N m=d n=S k=S, lda=H, ldb=S*A, ldc=H). */
+ * (gemm_batch N,N m=d n=S k=S, lda=H, ldb=S*A, ldc=H). */
 void oracle_att_qk_v(int batch, int seq_length, int heads, int size_per_head, const float *qk,
                      const float *value, float *out, float alpha, float beta) {
-    int S = seq_length, A = heads, d = size_per_head;
+    int S = seq_length, A = heads, d = size_per_head, count = batch * heads;
+    const float **v = (const float **) malloc(sizeof(float *) * (size_t) count);
+    const float **p = (const float **) malloc(sizeof(float *) * (size_t) count);
+    float **o = (float **) malloc(sizeof(float *) * (size_t) count);
     for (int b = 0; b < batch; ++b) {
         for (int h = 0; h < A; ++h) {
             size_t idx = (size_t) b * S * d * A + (size_t) d * h;
-            const float *p = qk + (size_t) b * S * S * A + (size_t) S * h;
-            oracle_sgemm(0, 0, d, S, S, alpha, value + idx, d * A, p, S * A, beta, out + idx,
-                         d * A);
+            v[b * A + h] = value + idx;
+            p[b * A + h] = qk + (size_t) b * S * S * A + (size_t) S * h;
+            o[b * A + h] = out + idx;
         }
     }
+    oracle_sgemm_batch(0, 0, d, S, S, alpha, v, d * A, p, S * A, beta, o, d * A, count);
+    free(o);
+    free(p);
+    free(v);
 }
 
 static const float *find_var(const oracle_vars *vars, const char *name) {
@@ -265,15 +337,15 @@ int oracle_attention_self(const oracle_vars *vars, const char *prefix, int batch
     float *q = falloc(M * H), *k = falloc(M * H), *v = falloc(M * H);
     float *scores = falloc((size_t) batch * A * S * S);
 
-    memcpy(scores, neg_mask, sizeof(float) * (size_t) batch * A * S * S);
-    oracle_dense((int) M, H, H, qk_, qb, in, q);
-    oracle_dense((int) M, H, H, kk, kb, in, k);
-    oracle_dense((int) M, H, H, vk, vb, in, v);
+    TIMED(ORACLE_PART_OTHER, memcpy(scores, neg_mask, sizeof(float) * (size_t) batch * A * S * S));
+    TIMED(ORACLE_PART_DENSE, oracle_dense((int) M, H, H, qk_, qb, in, q));
+    TIMED(ORACLE_PART_DENSE, oracle_dense((int) M, H, H, kk, kb, in, k));
+    TIMED(ORACLE_PART_DENSE, oracle_dense((int) M, H, H, vk, vb, in, v));
 
     float alpha = (float) (1.0 / sqrt((double) d));
-    oracle_att_q_k(batch, S, A, d, q, k, scores, alpha, -10000.0f);
-    oracle_softmax_(scores, scores, batch * A * S, S);
-    oracle_att_qk_v(batch, S, A, d, scores, v, context_out, 1.f, 0.f);
+    TIMED(ORACLE_PART_ATTENTION_GEMM, oracle_att_q_k(batch, S, A, d, q, k, scores, alpha, -10000.0f));
+    TIMED(ORACLE_PART_ROW_KERNELS, oracle_softmax_(scores, scores, batch * A * S, S));
+    TIMED(ORACLE_PART_ATTENTION_GEMM, oracle_att_qk_v(batch, S, A, d, scores, v, context_out, 1.f, 0.f));
 
     free(scores);
     free(v);
@@ -291,7 +363,7 @@ int oracle_transformer(const oracle_vars *vars, const char *prefix, int batch, i
     int rc = 0;
 
     float *neg_mask = falloc((size_t) batch * heads * S * S);
-    oracle_attention_mask(batch, S, heads, mask, neg_mask);
+    TIMED(ORACLE_PART_OTHER, oracle_attention_mask(batch, S, heads, mask, neg_mask));
 
     float *prev = falloc(M * H);
     memcpy(prev, in, sizeof(float) * M * H);
@@ -322,14 +394,14 @@ int oracle_transformer(const oracle_vars *vars, const char *prefix, int batch, i
         rc = oracle_attention_self(vars, ap, batch, S, heads, H / heads, prev, neg_mask, ctx);
         if (rc) break;
         /* attention/output: dense, then LayerNorm(residual = layer input) */
-        oracle_dense((int) M, H, H, aok, aob, ctx, att_out);
-        oracle_layer_norm_(prev, att_out, (int) M, H, anb, ang);
+        TIMED(ORACLE_PART_DENSE, oracle_dense((int) M, H, H, aok, aob, ctx, att_out));
+        TIMED(ORACLE_PART_ROW_KERNELS, oracle_layer_norm_(prev, att_out, (int) M, H, anb, ang));
         /* intermediate: dense + GELU */
-        oracle_dense((int) M, H, I, ik, ib, att_out, inter);
-        oracle_gelu(M * I, inter);
+        TIMED(ORACLE_PART_DENSE, oracle_dense((int) M, H, I, ik, ib, att_out, inter));
+        TIMED(ORACLE_PART_ROW_KERNELS, oracle_gelu(M * I, inter));
         /* output: dense, then LayerNorm(residual = attention output) */
-        oracle_dense((int) M, I, H, ok, ob, inter, layer_out);
-        oracle_layer_norm_(att_out, layer_out, (int) M, H, onb, ong);
+        TIMED(ORACLE_PART_DENSE, oracle_dense((int) M, I, H, ok, ob, inter, layer_out));
+        TIMED(ORACLE_PART_ROW_KERNELS, oracle_layer_norm_(att_out, layer_out, (int) M, H, onb, ong));
 
         float *t = prev;
         prev = layer_out;
@@ -412,7 +484,8 @@ int oracle_bert_forward(const oracle_vars *vars, int batch, int seq_length, int 
     float *emb = embedding_output ? embedding_output : falloc(M * H);
     float *seq = sequence_output ? sequence_output : falloc(M * H);
     float *pooled = pooled_output ? pooled_output : falloc((size_t) batch * H);
-    int rc = oracle_bert_embeddings(vars, batch, S, H, ids, segments, emb);
+    int rc;
+    TIMED(ORACLE_PART_OTHER, rc = oracle_bert_embeddings(vars, batch, S, H, ids, segments, emb));
     if (rc == 0) {
         rc = oracle_transformer(vars, "bert/encoder", batch, S, H, layers, heads, intermediate, emb,
                                 mask, seq);

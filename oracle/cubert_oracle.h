@@ -15,6 +15,7 @@
  *   oracle_not                  reference AttentionMaskTest vector; reference op build
  *   oracle_tanh_, oracle_reduce_mean_1   reference BertPoolerTest vectors; reference op build
  *   oracle_sgemm                reference DenseTest / BatchMatMulTest integer vectors; numpy float64 matmul
+ *   oracle_sgemm_batch          through oracle_att_q_k / qk_v: reference BatchMatMulTest vectors, both batch modes
  *   oracle_dense                reference DenseTest vector
  *   oracle_attention_mask       reference AttentionMaskTest vector (24 values)
  *   oracle_att_q_k / qk_v       reference BatchMatMulTest vectors
@@ -49,6 +50,22 @@ const char *oracle_blas_name(void);
 void oracle_sgemm(int transA, int transB, int M, int N, int K, float alpha,
                   const float *A, int lda, const float *B, int ldb, float beta,
                   float *C, int ldc);
+
+/* One group of `count` independent column-major sgemm problems of one shape, cblas_sgemm_batch's meaning.
+ * reference: src/cuBERT/common.cpp:260-298 (blas_gemm_batch<float>, HAVE_MKL branch). */
+void oracle_sgemm_batch(int transA, int transB, int M, int N, int K, float alpha, const float **A, int lda,
+                        const float **B, int ldb, float beta, float **C, int ldc, int count);
+/* on (default): the problems of a batch run as an OpenMP loop around single-threaded sgemm calls, which is how
+ * MKL's cblas_sgemm_batch spreads a group; off: one multi-threaded sgemm after the other.  Same results. */
+void oracle_set_batch_parallel(int on);
+/* Thread count the loaded BLAS reports for itself (0 for the builtin loop, which follows OpenMP). */
+int oracle_blas_threads(void);
+
+/* Wall-clock seconds spent per part of oracle_bert_forward / oracle_transformer since the last reset. */
+enum { ORACLE_PART_DENSE = 0, ORACLE_PART_ATTENTION_GEMM = 1, ORACLE_PART_ROW_KERNELS = 2, ORACLE_PART_OTHER = 3,
+       ORACLE_PROFILE_PARTS = 4 };
+void oracle_profile_reset(void);
+void oracle_profile_read(double seconds[ORACLE_PROFILE_PARTS]);
 
 /* ---- primitive ops (reference: src/cuBERT/op, op_att, op_bert) ---------- */
 

@@ -181,13 +181,22 @@ def test_benchmark_configurations(cb, name, rows):
     for k in ("pooled_output", "logits", "probs") + (() if half else ("sequence_output", "embedding_output")):
         report[k] = assert_close(got[k][:n], want[k], tol, "%s %s" % (name, k))
     if half:
-        # token-level outputs of the fp16 path, absolute, as the reference bounds them: embedding output 3e-4 ... 2e-3
-        # (BertTest.cpp:96-101), encoder output 1e-3 ... 1e-2 (TransformerTest.cpp:330-341)
-        for k, bound in (("embedding_output", 2e-3), ("sequence_output", 1e-2)):
+        # Token-level outputs of the fp16 path, element by element, with the reference's own absolute tolerances for
+        # outputs of order 1: 3e-4 on the embedding output (BertTest.cpp:96-101; its 2e-3 is for one larger element)
+        # and 1e-2 on the encoder output (TransformerTest.cpp:330-341).  LayerNorm outputs of 768 ... 1024 channels
+        # reach 5 ... 9, where one fp16 rounding alone is up to 2^-11 |x| (2e-3 at 4, 3.9e-3 at 8), so the embedding
+        # bound carries that term and the encoder bound scales with elements above 1.
+        d = {k: np.abs(got[k][:n].astype(np.float64) - want[k]) for k in ("embedding_output", "sequence_output")}
+        size = {k: np.abs(want[k]) for k in d}
+        assert (d["embedding_output"] <= 3e-4 + size["embedding_output"] * 2.0 ** -11).all(), \
+            (name, float((d["embedding_output"] - size["embedding_output"] * 2.0 ** -11).max()))
+        assert (d["sequence_output"] <= 1e-2 * np.maximum(1.0, size["sequence_output"])).all(), \
+            (name, float((d["sequence_output"] / np.maximum(1.0, size["sequence_output"])).max()))
+        for k in d:
             report[k] = rel_err(got[k][:n], want[k])
-            worst = float(np.abs(got[k][:n].astype(np.float64) - want[k]).max())
-            report[k + " (abs)"] = worst
-            assert worst <= bound, (name, k, worst)
+            report[k + " (abs)"] = float(d[k].max())
+            report[k + " (rms)"] = float(np.sqrt((d[k] ** 2).mean()))
+            report[k + " (largest)"] = float(size[k].max())
     print("\n%s relative errors vs oracle: %s" % (name, {k: "%.2e" % v for k, v in report.items()}))
     # size-independent properties at the full batch
     np.testing.assert_allclose(got["probs"].sum(-1), 1.0, atol=2e-3 if half else 1e-5)

@@ -57,13 +57,29 @@ def test_attention_mask_vector(case):
     assert c.check(out) == 24
 
 
-def test_batch_matmul_vectors(case):
-    c = case(T + "op_att/BatchMatMulTest.cpp", "q_k")
-    out = oracle.att_q_k(c.arrays["query"], c.arrays["key"], 2, 2, 4, 3)
-    assert c.check(out) == 32
-    c = case(T + "op_att/BatchMatMulTest.cpp", "qk_v")
-    out = oracle.att_qk_v(c.arrays["qk"], c.arrays["value"], 2, 2, 4, 3)
-    assert c.check(out) == 48
+@pytest.mark.parametrize("blas,batch_parallel", [("builtin", True), ("best", True), ("best", False)])
+def test_batch_matmul_vectors(case, blas, batch_parallel):
+    """The pointer-array batch (one cblas_sgemm_batch group in the reference) with the builtin loop, as an OpenMP
+    loop around single-threaded BLAS calls, and as one multi-threaded BLAS call per problem."""
+    oracle.use_builtin_gemm() if blas == "builtin" else oracle.use_best_blas()
+    oracle.set_batch_parallel(batch_parallel)
+    try:
+        c = case(T + "op_att/BatchMatMulTest.cpp", "q_k")
+        out = oracle.att_q_k(c.arrays["query"], c.arrays["key"], 2, 2, 4, 3)
+        assert c.check(out) == 32
+        c = case(T + "op_att/BatchMatMulTest.cpp", "qk_v")
+        out = oracle.att_qk_v(c.arrays["qk"], c.arrays["value"], 2, 2, 4, 3)
+        assert c.check(out) == 48
+        # the two batch modes are the same sgemm per problem: equal bits at a BERT-base head shape
+        rng = np.random.default_rng(3)
+        q, k = (rng.normal(size=(3 * 32 * 12 * 64)).astype(np.float32) for _ in range(2))
+        a = oracle.att_q_k(q, k, 3, 32, 12, 64, alpha=0.125)
+        oracle.set_batch_parallel(not batch_parallel)
+        b = oracle.att_q_k(q, k, 3, 32, 12, 64, alpha=0.125)
+        assert np.array_equal(a, b)
+    finally:
+        oracle.set_batch_parallel(True)
+        oracle.use_best_blas()
 
 
 def test_attention_self_vector(case):
