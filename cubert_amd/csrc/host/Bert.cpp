@@ -1,8 +1,10 @@
 #include "Bert.h"
 
+#include <cstdlib>
 #include <cstring>
 #include <iostream>
 #include <stdexcept>
+#include <string>
 #include <vector>
 
 namespace cuBERT {
@@ -86,6 +88,9 @@ Bert<T>::Bert(const std::unordered_map<std::string, T *> &var, size_t max_batch_
         if (input_staging == nullptr) throw std::runtime_error("no page-locked host memory for the request inputs");
         output_staging = static_cast<unsigned char *>(cubert_malloc_host(kOutputStagingBytes));
         if (output_staging == nullptr) throw std::runtime_error("no page-locked host memory for the outputs");
+
+        const char *warm = std::getenv("CUBERT_OPEN_WARMUP");
+        if (warm == nullptr || std::string(warm) != "0") _pre_compute(max_batch_size);
     } catch (...) {
         release();
         throw;
@@ -133,8 +138,31 @@ void Bert<T>::layout_buffers() {
     _probs = has_classifier ? buffers.take<T>(max_batch_size * num_labels) : nullptr;
 }
 
+// What a first request of `batch_size` sequences would otherwise pay for: one forward pass on made-up inputs, so
+// that every GEMM shape of that batch size is planned and, where that applies, its algorithm chosen by timing
+// (tens of milliseconds) before a caller waits on it.  The reference also prepares the maximum batch when a model
+// is built (src/cuBERT/Bert.cpp:62-64, there: bias rows copied into the Dense outputs).  Other batch sizes are
+// still planned on their first request.
 template <typename T>
-void Bert<T>::_pre_compute(size_t) {}
+void Bert<T>::_pre_compute(size_t batch_size) {
+    if (batch_size == 0 || batch_size > max_batch_size || vocab_size == 0) return;
+    const size_t M = batch_size * seq_length;
+    const size_t mask_at = round_up_16(sizeof(int) * M), segments_at = round_up_16(mask_at + M);
+    if (input_copy_pending) synchronize();
+    // ids spread over the vocabulary (a multiplicative hash of the position), every position valid, segment 0:
+    // activations like those of a real request, which is what the timing of GEMM algorithms should see
+    int *ids = reinterpret_cast<int *>(input_staging);
+    for (size_t i = 0; i < M; ++i) ids[i] = (int) ((uint32_t) (i * 2654435761u) % (uint32_t) vocab_size);
+    std::memset(input_staging + mask_at, 1, M);
+    std::memset(input_staging + segments_at, 0, M);
+    cuBERT::memcpyAsync(input_block, input_staging, segments_at + M, 1, stream);
+    input_ids_buf = reinterpret_cast<int *>(input_block);
+    input_mask_buf = reinterpret_cast<int8_t *>(input_block + mask_at);
+    segment_ids_buf = reinterpret_cast<int8_t *>(input_block + segments_at);
+    forward(batch_size);
+    synchronize();
+    input_ids_buf = nullptr, input_mask_buf = nullptr, segment_ids_buf = nullptr;  // no request is resident
+}
 
 template <typename T>
 void Bert<T>::synchronize() {

@@ -37,7 +37,10 @@ public:
     Bert(const Bert &) = delete;
     Bert &operator=(const Bert &) = delete;
 
-    // Nothing to prepare between requests in this implementation; kept so callers of the reference compile.
+    // One forward pass of `batch_size` sequences on made-up inputs: plans (and where it applies times) every GEMM
+    // shape of that batch size, so that the first request of that size does not pay for it.  The constructor runs
+    // it for max_batch_size (CUBERT_OPEN_WARMUP=0 in the environment skips that).  Nothing needs preparing
+    // between requests, unlike in the reference, whose _pre_compute refills the Dense outputs with their biases.
     void _pre_compute(size_t batch_size);
 
     // Copies the three host input arrays to the device and enqueues the forward pass.  Asynchronous:

@@ -192,26 +192,7 @@ __global__ __launch_bounds__(kBlock) void ln_pair_kernel(T *__restrict__ inout, 
     const bool has_second = row0 + 1 < rows;  // wavefront-uniform
     const bool upper = lane >= 32;            // in load 1 the upper half of the lanes belongs to the second row
 
-    // wavefront-uniform row bases (scalar loads for the ids)
-    const T *src_a[2], *src_b[2], *src_c[2];
-    if (EMBED) {
-#pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            const int row = (k == 1 && !has_second) ? row0 : row0 + k;
-            src_a[k] = word + (size_t) ids[row] * H;
-            src_b[k] = pos + (size_t) (row % seq_length) * H;
-            src_c[k] = type + (size_t) segments[row] * H;
-        }
-    } else {
-#pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            src_a[k] = inout + (size_t) (row0 + k) * H;
-            src_b[k] = bias;
-            src_c[k] = residual + (size_t) (row0 + k) * H;
-        }
-    }
     T *dst[1] = {inout + (size_t) row0 * H};
-
     Vec<T, VEC> a[3], b[3], c[3], g[3], be[3];
     int col[3];
     bool second[3], active[3];
@@ -221,25 +202,54 @@ __global__ __launch_bounds__(kBlock) void ln_pair_kernel(T *__restrict__ inout, 
         second[k] = k == 2 || (k == 1 && upper);
         col[k] = second[k] ? flat - H : flat;
         active[k] = !second[k] || has_second;
-        // Loads are unconditional (a lane whose row does not exist re-reads the first row and is masked out of
-        // the sums and the stores below), so nothing stands between the loads of a wavefront.
-        if (EMBED) {
-            const bool from_second = second[k] && has_second;
-            a[k] = load_vec<T, VEC>((from_second ? src_a[1] : src_a[0]) + col[k]);
-            c[k] = load_vec<T, VEC>((from_second ? src_c[1] : src_c[0]) + col[k]);
-            b[k] = load_vec<T, VEC>((from_second ? src_b[1] : src_b[0]) + col[k]);
-        } else {
-            // the two rows are adjacent in memory: one base address, the offset inside the two-row span
-            const int at = active[k] ? flat : col[k];
-            a[k] = load_vec<T, VEC>(src_a[0] + at);
-            c[k] = load_vec<T, VEC>(src_c[0] + at);
-        }
     }
+    // Loads are unconditional (a lane whose row does not exist re-reads the first row and is masked out of the
+    // sums and the stores below), so nothing stands between the loads of a wavefront.
+    if (EMBED) {
+        // Wavefront-uniform ids through scalar loads: both rows' ids in one 8-byte load where the pair is aligned
+        // (row0 is even), the segment ids as the aligned words that hold them.  The loads that do not depend on
+        // them (position rows, gamma, beta) are issued while the ids are on their way.
+        const int row1 = has_second ? row0 + 1 : row0;
+        int id0, id1;
+        if (has_second && is_aligned(ids + row0, 8)) {
+            const int2 both = *reinterpret_cast<const int2 *>(ids + row0);
+            id0 = both.x;
+            id1 = both.y;
+        } else {
+            id0 = ids[row0];
+            id1 = ids[row1];
+        }
+        const int seg0 = uniform_i8(segments, row0), seg1 = uniform_i8(segments, row1);
+        const T *pos0 = pos + (size_t) (row0 % seq_length) * H, *pos1 = pos + (size_t) (row1 % seq_length) * H;
 #pragma unroll
-    for (int k = 0; k < 3; ++k) {
-        if (!EMBED && HAS_BIAS) b[k] = load_vec<T, VEC>(bias + col[k]);
-        g[k] = load_vec<T, VEC>(gamma + col[k]);
-        be[k] = load_vec<T, VEC>(beta + col[k]);
+        for (int k = 0; k < 3; ++k) {
+            b[k] = load_vec<T, VEC>((second[k] ? pos1 : pos0) + col[k]);
+            g[k] = load_vec<T, VEC>(gamma + col[k]);
+            be[k] = load_vec<T, VEC>(beta + col[k]);
+        }
+        asm volatile("" ::: "memory");
+        const T *word0 = word + (size_t) id0 * H, *word1 = word + (size_t) id1 * H;
+        const T *type0 = type + (size_t) seg0 * H, *type1 = type + (size_t) seg1 * H;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            a[k] = load_vec<T, VEC>((second[k] ? word1 : word0) + col[k]);
+            c[k] = load_vec<T, VEC>((second[k] ? type1 : type0) + col[k]);
+        }
+    } else {
+        // the two rows are adjacent in memory: one base address, the offset inside the two-row span
+        const T *gemm_out = inout + (size_t) row0 * H, *res = residual + (size_t) row0 * H;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const int at = active[k] ? (k * kWave + lane) * VEC : col[k];
+            a[k] = load_vec<T, VEC>(gemm_out + at);
+            c[k] = load_vec<T, VEC>(res + at);
+        }
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            if (HAS_BIAS) b[k] = load_vec<T, VEC>(bias + col[k]);
+            g[k] = load_vec<T, VEC>(gamma + col[k]);
+            be[k] = load_vec<T, VEC>(beta + col[k]);
+        }
     }
     // every load above is issued before the first conversion below (loads do not move across this point)
     asm volatile("" ::: "memory");

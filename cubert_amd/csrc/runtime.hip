@@ -90,6 +90,7 @@ struct BlasContext {
     int *skinny_counters = nullptr;  // zero between launches (the kernel resets what it counted)
     std::map<GemmKey, GemmPlan> plans;
     std::mutex mutex;
+    bool used = false;  // something was launched on `stream` since it was set
 };
 
 #define LT_TRY(call)                                                                                      \
@@ -336,6 +337,14 @@ int run_skinny(BlasContext *ctx, int type, int M, int N, int K, float alpha, con
                                                ctx->stream);
 }
 
+// The same for the entry points that reach the kernel directly: one launch at a time per context.
+int run_skinny_locked(BlasContext *ctx, int type, int M, int N, int K, float alpha, const void *A, int lda,
+                      const void *B, int ldb, void *C, int ldc, const void *bias, int activation, int packed = 0) {
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    ctx->used = true;
+    return run_skinny(ctx, type, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, activation, packed);
+}
+
 int run_gemm(void *handle, int type, int transA, int transB, int M, int N, int K, float alpha, const void *A, int lda,
              long long strideA, const void *B, int ldb, long long strideB, float beta, void *C, int ldc,
              long long strideC, int batch, const void *bias) {
@@ -344,15 +353,17 @@ int run_gemm(void *handle, int type, int transA, int transB, int M, int N, int K
     if (M == 0 || N == 0 || batch == 0) return 0;
     GemmKey key{type, transA, transB, M, N, K, lda, ldb, ldc, batch, strideA, strideB, strideC, bias != nullptr,
                 beta == 0.f};
+    ctx->used = true;
     if (force_naive_gemm()) {
         return run_naive_gemm(ctx->stream, type, transA, transB, M, N, K, alpha, A, lda, strideA, B, ldb, strideB,
                               beta, C, ldc, strideC, batch, bias);
     }
+    // one launch at a time per context: the plan cache, and the few-token kernel's partial tiles and counters
+    std::lock_guard<std::mutex> lock(ctx->mutex);
     if (type != 2 && !transA && !transB && batch == 1 && beta == 0.f && N <= 32 && !library_gemm_only()) {
         const int rc = run_skinny(ctx, type, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, 0);
         if (rc != CUBERT_UNSUPPORTED) return rc;
     }
-    std::lock_guard<std::mutex> lock(ctx->mutex);
     auto it = ctx->plans.find(key);
     if (it == ctx->plans.end()) {
         GemmPlan plan;
@@ -512,7 +523,16 @@ int cubert_blas_destroy(void *handle) {
 
 int cubert_blas_set_stream(void *handle, void *stream) {
     if (!handle) return CUBERT_BAD_ARGUMENT;
-    ((BlasContext *) handle)->stream = (hipStream_t) stream;
+    BlasContext *ctx = (BlasContext *) handle;
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    if (ctx->stream != (hipStream_t) stream && ctx->used) {
+        // launches on the old stream may still be using the context's workspaces: let them finish before the
+        // next launch, on the new stream, reuses them
+        const int rc = hip_rc(hipStreamSynchronize(ctx->stream));
+        if (rc) return rc;
+        ctx->used = false;
+    }
+    ctx->stream = (hipStream_t) stream;
     return 0;
 }
 
@@ -539,7 +559,7 @@ int cubert_gemm_skinny_f32(void *handle, int M, int N, int K, float alpha, const
     BlasContext *ctx = (BlasContext *) handle;
     if (!ctx || !A || !B || !C) return CUBERT_BAD_ARGUMENT;
     if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;
-    return run_skinny(ctx, 0, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, activation);
+    return run_skinny_locked(ctx, 0, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, activation);
 }
 
 int cubert_gemm_skinny_f16(void *handle, int M, int N, int K, float alpha, const cubert_half *A, int lda,
@@ -548,7 +568,7 @@ int cubert_gemm_skinny_f16(void *handle, int M, int N, int K, float alpha, const
     BlasContext *ctx = (BlasContext *) handle;
     if (!ctx || !A || !B || !C) return CUBERT_BAD_ARGUMENT;
     if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;
-    return run_skinny(ctx, 1, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, activation);
+    return run_skinny_locked(ctx, 1, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, activation);
 }
 
 size_t cubert_gemm_skinny_packed_elements(int M, int K) { return cubert::gemm_skinny_packed_elements(M, K); }
@@ -571,7 +591,7 @@ int cubert_gemm_skinny_packed_f32(void *handle, int M, int N, int K, float alpha
     BlasContext *ctx = (BlasContext *) handle;
     if (!ctx || !packedA || !B || !C) return CUBERT_BAD_ARGUMENT;
     if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;
-    return run_skinny(ctx, 0, M, N, K, alpha, packedA, 0, B, ldb, C, ldc, bias, activation, 1);
+    return run_skinny_locked(ctx, 0, M, N, K, alpha, packedA, 0, B, ldb, C, ldc, bias, activation, 1);
 }
 
 int cubert_gemm_skinny_packed_f16(void *handle, int M, int N, int K, float alpha, const cubert_half *packedA,
@@ -580,7 +600,7 @@ int cubert_gemm_skinny_packed_f16(void *handle, int M, int N, int K, float alpha
     BlasContext *ctx = (BlasContext *) handle;
     if (!ctx || !packedA || !B || !C) return CUBERT_BAD_ARGUMENT;
     if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;
-    return run_skinny(ctx, 1, M, N, K, alpha, packedA, 0, B, ldb, C, ldc, bias, activation, 1);
+    return run_skinny_locked(ctx, 1, M, N, K, alpha, packedA, 0, B, ldb, C, ldc, bias, activation, 1);
 }
 
 int cubert_gemm_strided_batch_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha,

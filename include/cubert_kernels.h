@@ -198,7 +198,13 @@ int cubert_event_elapsed_ms(void *start, void *stop, float *ms); /* both events 
  * kernel's execution time alone.  One shot: cleared by the launch.  NULL, NULL cancels. */
 int cubert_time_next_launch(void *start_event, void *stop_event);
 
-/* A BLAS context: a hipBLASLt handle, a workspace, a plan cache, bound to one stream. */
+/* A BLAS context: a hipBLASLt handle, a workspace, a plan cache and the few-token kernel's scratch (partial tiles
+ * and arrival counters), bound to one stream.  One set of each per context, so a context's GEMMs belong on ONE
+ * stream and come from one thread at a time: the library serialises the calls of several threads on one handle
+ * (a mutex), and cubert_blas_set_stream to a different stream first waits for what the context launched on the
+ * old one, but launches of one context never overlap on the device.  Callers that want GEMMs to overlap use one
+ * context per stream (as Bert<T> does: one context and one stream per model instance, the reference's
+ * arrangement, src/cuBERT/Bert.cpp:23-25). */
 void *cubert_blas_create(void);
 int cubert_blas_destroy(void *handle);
 int cubert_blas_set_stream(void *handle, void *stream);
@@ -260,8 +266,9 @@ int cubert_bias_res_ln_split3_f32(float *inout, const float *residual, const flo
  * of 16 and B 16-byte aligned with ldb a multiple of 16 bytes; anything else returns CUBERT_UNSUPPORTED and
  * launches nothing (also with CUBERT_GEMM=library or naive in the environment).  activation: 0 = none, 1 = the
  * erf-form GELU of cubert_bias_gelu applied to the result (Dense + bias + GELU of BertIntermediate in one
- * launch; reference src/cuBERT/op_att/Transformer.cpp:164-165).  Calls on one handle must not overlap (they share
- * the handle's scratch).
+ * launch; reference src/cuBERT/op_att/Transformer.cpp:164-165).  Launches of one handle share its partial-tile
+ * workspace and counters and are ordered by the handle's one stream (see cubert_blas_create); they never run
+ * concurrently.
  * replaces: Dense<T>::compute -> blas_gemm<T> for small batch * seq_length, reference
  * src/cuBERT/op/Dense.cpp:47-57 (bias: Dense.cpp:41-44). */
 int cubert_gemm_skinny_f32(void *handle, int M, int N, int K, float alpha, const float *A, int lda, const float *B,

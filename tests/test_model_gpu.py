@@ -407,6 +407,31 @@ def test_models_per_gpu_must_be_a_sane_count(cb, small_pb, monkeypatch):
             cb.Model(path, 4, 32, 3, 4)
 
 
+def test_first_request_does_not_pay_for_gemm_planning(cb):
+    """The constructor runs one forward pass at max_batch_size (Bert<T>::_pre_compute), so the GEMM shapes of that
+    batch size are planned and timed before the first request: BERT-base width, 2 layers, batch 128 x seq 32 (Dense
+    GEMMs of 4.8 ... 19 GFLOP, the size whose algorithms are chosen by timing 32 candidates)."""
+    import time
+    from cubert_amd.testing import BERT_BASE, random_bert_weights, random_inputs
+    shape = dict(BERT_BASE, layers=2, vocab=1000, max_position=32)
+    w = random_bert_weights(seed=5, labels=2, **shape)
+    ids, mask, seg = random_inputs(seed=6, batch=128, seq_length=32, vocab=1000, min_valid=8)
+    bert = cb.Bert(w, 128, 32, 2, 12)
+    out = cb.Output(np.empty((128, 768), np.float32), cb.OutputType.POOLED_OUTPUT)
+    times = []
+    for _ in range(6):
+        t = time.perf_counter()
+        bert.compute(ids, mask, seg)
+        bert.output(128, out)
+        times.append((time.perf_counter() - t) * 1e3)
+    bert.close()
+    later = float(np.median(times[1:]))
+    print("\nfirst request %.2f ms, later requests %.2f ms (median of 5)" % (times[0], later))
+    assert times[0] <= 3 * later + 2.0, times
+    want = oracle.bert_forward(w, ids[:4], mask[:4], seg[:4], 2, 12)["pooled_output"]
+    assert_close(out.pooled_output[:4], want, FP32_TOL, "pooled output after the timed requests")
+
+
 def test_api_error_behaviour(cb, small_pb):
     path, _ = small_pb
     with pytest.raises(ValueError, match="model file not found"):
