@@ -92,6 +92,7 @@ SIGNATURES = {
     "cubert_event_record": (ci, [vp, vp]),
     "cubert_event_elapsed_ms": (ci, [vp, vp, ctypes.POINTER(cf)]),
     "cubert_time_next_launch": (ci, [vp, vp]),
+    "cubert_gemm_skinny_noalloc_f32": (ci, [vp, ci, ci, ci, cf, vp, ci, vp, ci, vp, ci, vp, ci]),
     "cubert_gemm_skinny_packed_elements": (ctypes.c_size_t, [ci, ci]),
     "cubert_gemm_f16_f32": (ci, [vp, ci, ci, ci, ci, ci, cf, vp, ci, vp, ci, cf, vp, ci, vp]),
     "cubert_split3_f32": (ci, [vp, ci, ci, cf, ci, vp, vp]),

@@ -15,6 +15,9 @@
 // workspace and the last workgroup to arrive for a feature block (ticket from an atomic counter) adds the
 // slices in slice order, so the result does not depend on scheduling.
 
+#include <cstdio>
+#include <mutex>
+
 #include "activations.h"
 #include "cubert_kernels.h"
 #include "device_common.h"
@@ -222,6 +225,84 @@ int gemm_skinny_pack(const T *A, int lda, int M, int K, T *packed, hipStream_t s
     if (blocks > 0x7fffffffull) return CUBERT_UNSUPPORTED;
     return launch(gemm_skinny_pack_kernel<T>, dim3((unsigned) blocks), dim3(kBlock), stream, A, lda, M,
                   K / kSkinnyChunk, packed, total);
+}
+
+// ---- the same kernel for callers that cannot allocate ---------------------------------------------------
+// The split-K partial tiles and the arrival counters of cubert_gemm_skinny_noalloc_f32 live in this array, which is
+// part of the library's device image: each GPU the library runs on holds its own copy (4 MiB + 16 KiB) at its own
+// address until the process ends.  In host code the array's name is only a stand-in for the symbol; the device
+// address comes from hipGetSymbolAddress, once per device, and only that pointer is handed to kernels.
+namespace {
+
+constexpr size_t kNoAllocPartialFloats = 1u << 20;  // as many as a BLAS context's workspace: same K slices, same sums
+constexpr int kNoAllocCounters = 4096;
+constexpr size_t kNoAllocBytes = kNoAllocPartialFloats * sizeof(float) + kNoAllocCounters * sizeof(int);
+constexpr int kNoAllocMaxDevices = 64;
+
+// (`used`: no kernel names the array, every kernel receives its address as an argument)
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kNoAllocBytes];
+
+std::mutex g_noalloc_mutex;
+void *g_noalloc_scratch[kNoAllocMaxDevices];  // per device: address of that device's copy of `scratch`, once known
+
+__global__ __launch_bounds__(kBlock) void zero_ints_kernel(int *p, int n) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+// Address of the current device's copy of the array (looked up on the first call per device).
+int noalloc_scratch(unsigned char **out) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return (int) e;
+    if (device < 0 || device >= kNoAllocMaxDevices) {
+        fprintf(stderr, "cubert_gemm_skinny_noalloc_f32: device %d is outside the %d devices it keeps scratch addresses for\n",
+                device, kNoAllocMaxDevices);
+        return CUBERT_BAD_ARGUMENT;
+    }
+    std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+    if (g_noalloc_scratch[device] == nullptr) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) {
+            fprintf(stderr, "cubert_gemm_skinny_noalloc_f32: hipGetSymbolAddress failed on device %d: %s\n", device,
+                    hipGetErrorString(e));
+            return e != hipSuccess ? (int) e : CUBERT_BAD_ARGUMENT;
+        }
+        g_noalloc_scratch[device] = ptr;
+    }
+    *out = static_cast<unsigned char *>(g_noalloc_scratch[device]);
+    return 0;
+}
+
+}  // namespace
+
+int gemm_skinny_noalloc_f32(int M, int N, int K, float alpha, const float *A, int lda, const float *B, int ldb, float *C,
+                            int ldc, const float *bias, int activation, hipStream_t stream) {
+    if (!A || !B || !C) return CUBERT_BAD_ARGUMENT;
+    if (M > CUBERT_GEMM_SKINNY_NOALLOC_MAX_M || K > CUBERT_GEMM_SKINNY_NOALLOC_MAX_K) {
+        fprintf(stderr,
+                "cubert_gemm_skinny_noalloc_f32: M = %d, K = %d is beyond what its fixed scratch array is sized for "
+                "(M <= %d output features, K <= %d); use cubert_gemm_skinny_f32 with a BLAS context\n",
+                M, K, CUBERT_GEMM_SKINNY_NOALLOC_MAX_M, CUBERT_GEMM_SKINNY_NOALLOC_MAX_K);
+        return CUBERT_TOO_LARGE;
+    }
+    unsigned char *base = nullptr;
+    const int rc = noalloc_scratch(&base);
+    if (rc) return rc;
+    float *partials = reinterpret_cast<float *>(base);
+    int *counters = reinterpret_cast<int *>(base + kNoAllocPartialFloats * sizeof(float));
+    // The array keeps what the last call left in it.  The partial tiles are written before they are read; the
+    // counters must start at zero, so the ones this launch can touch are cleared first, on the same stream, by a
+    // kernel (not a memset node, which a caller's graph capture would record).
+    const int blocks = M > 0 ? (M + 31) / 32 : 0;
+    if (blocks > 0 && blocks <= kNoAllocCounters) {
+        const int e = launch_untimed(zero_ints_kernel, dim3((blocks + kBlock - 1) / kBlock), dim3(kBlock), 0, stream,
+                                     counters, blocks);
+        if (e) return e;
+    }
+    return gemm_skinny<float>(M, N, K, alpha, A, lda, 0, B, ldb, C, ldc, bias, activation, partials,
+                              kNoAllocPartialFloats, counters, kNoAllocCounters, stream);
 }
 
 template int gemm_skinny<float>(int, int, int, float, const float *, int, int, const float *, int, float *, int,

@@ -28,6 +28,8 @@ int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, int packe
                 const T *bias, int activation, float *partials, size_t partial_floats, int *counters,
                 int n_counters, hipStream_t stream);
 size_t gemm_skinny_packed_elements(int M, int K);
+int gemm_skinny_noalloc_f32(int M, int N, int K, float alpha, const float *A, int lda, const float *B, int ldb, float *C,
+                            int ldc, const float *bias, int activation, hipStream_t stream);
 template <typename T>
 int gemm_skinny_pack(const T *A, int lda, int M, int K, T *packed, hipStream_t stream);
 
@@ -569,6 +571,12 @@ int cubert_gemm_skinny_f16(void *handle, int M, int N, int K, float alpha, const
     if (!ctx || !A || !B || !C) return CUBERT_BAD_ARGUMENT;
     if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;
     return run_skinny_locked(ctx, 1, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, activation);
+}
+
+int cubert_gemm_skinny_noalloc_f32(void *stream, int M, int N, int K, float alpha, const float *A, int lda,
+                                   const float *B, int ldb, float *C, int ldc, const float *bias, int activation) {
+    return cubert::gemm_skinny_noalloc_f32(M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, activation,
+                                           (hipStream_t) stream);
 }
 
 size_t cubert_gemm_skinny_packed_elements(int M, int K) { return cubert::gemm_skinny_packed_elements(M, K); }

@@ -33,6 +33,7 @@ extern "C" {
 typedef uint16_t cubert_half;
 #define CUBERT_BAD_ARGUMENT (-1)
 #define CUBERT_UNSUPPORTED (-2) /* valid arguments, but no kernel for this shape: the caller takes another route */
+#define CUBERT_TOO_LARGE (-3)   /* beyond the fixed capacity of an entry point that allocates nothing */
 
 /* ------------------------------------------------------------------ kernels */
 
@@ -276,6 +277,22 @@ int cubert_gemm_skinny_f32(void *handle, int M, int N, int K, float alpha, const
 int cubert_gemm_skinny_f16(void *handle, int M, int N, int K, float alpha, const cubert_half *A, int lda,
                            const cubert_half *B, int ldb, cubert_half *C, int ldc, const cubert_half *bias,
                            int activation);
+
+/* cubert_gemm_skinny_f32 for callers that cannot allocate device memory or hold a BLAS context: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference
+ * (whose GEMMs all go through a cuBLAS handle) and none is needed by the host classes here.  Same kernel, same
+ * arguments and return codes, same results bit for bit; instead of a handle it takes the stream, and the split-K
+ * partial tiles and arrival counters live in a fixed array inside the library's device image (4 MiB + 16 KiB on
+ * every GPU the library runs on, until the process ends).  The call allocates and frees nothing.  The array's
+ * size fixes the largest problem: M <= CUBERT_GEMM_SKINNY_NOALLOC_MAX_M output features and
+ * K <= CUBERT_GEMM_SKINNY_NOALLOC_MAX_K; beyond that CUBERT_TOO_LARGE is returned, a message goes to stderr and
+ * nothing is launched.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams,
+ * two threads) race on it; keep them on one stream or order them yourself.  The first call on a device looks up
+ * the array's address there (hipGetSymbolAddress), which is the only set-up. */
+#define CUBERT_GEMM_SKINNY_NOALLOC_MAX_M 32768
+#define CUBERT_GEMM_SKINNY_NOALLOC_MAX_K 65536
+int cubert_gemm_skinny_noalloc_f32(void *stream, int M, int N, int K, float alpha, const float *A, int lda,
+                                   const float *B, int ldb, float *C, int ldc, const float *bias, int activation);
 
 /* The few-token kernel on weights re-ordered once into the order it consumes them (a workgroup then streams
  * one contiguous run with 16-byte loads instead of 128-byte pieces at a stride of a weight row).
