@@ -249,15 +249,22 @@ def cpu_baseline(workload, cfg, w, ids, mask, seg):
                 "ms_per_pass": round(float(np.mean(times)) * 1e3, 1), "ms_per_pass_by_part": parts,
                 "threads": oracle.threads_in_use()}
 
-    main_leg = leg(default_threads, 3, 20)
-    four = leg(4, 2, 10) if default_threads > 4 else None
+    # The box's CPU share may be smaller than the logical CPUs it shows, and then a full team of spinning OpenMP
+    # threads is slower than a small one: the baseline is the best of the default team, half of it and 4 threads
+    # (the reference's CI setting), and every leg is reported.
+    counts = [default_threads] + [t for t in (default_threads // 2, 4) if 1 <= t < default_threads]
+    counts = sorted(set(counts), reverse=True)
+    legs = {t: leg(t, 3 if t == default_threads else 2, 12 if t == default_threads else 8) for t in counts}
     oracle.set_blas_threads(default_threads)
     if gomp is not None:
         gomp.omp_set_num_threads(default_threads)
+    best = max(legs, key=lambda t: legs[t]["value"])
+    main_leg = legs[best]
+    four = legs.get(4)
     dense = main_leg["ms_per_pass_by_part"]["dense_gemm"]
     M, H, I = n * S, m["hidden"], m["intermediate"]
     dense_flop = 2.0 * M * (4 * H * H + 2 * H * I) * m["layers"]
-    return {"value": main_leg["value"], "unit": "sequences/s", "cores": default_threads, "kind": "port",
+    return {"value": main_leg["value"], "unit": "sequences/s", "cores": best, "kind": "port",
             "sample": "%d pass(es) of %d sequences of %s (seq_len %d), fp32, mean %.1f ms/pass" %
                       (main_leg["passes"], n, workload, S, main_leg["ms_per_pass"]),
             "blas": os.path.basename(oracle.blas_name()),
@@ -265,7 +272,8 @@ def cpu_baseline(workload, cfg, w, ids, mask, seg):
                      "single-threaded sgemm calls, the way cblas_sgemm_batch spreads a group)",
             "threads": main_leg["threads"], "ms_per_pass_by_part": main_leg["ms_per_pass_by_part"],
             "dense_gemm_GFLOPs": round(dense_flop / (dense * 1e-3) / 1e9, 1) if dense > 0 else None,
-            "value_at_4_threads": four["value"] if four else None, "at_4_threads": four}
+            "value_at_4_threads": four["value"] if four else None,
+            "legs": {"%d threads" % t: legs[t] for t in counts}}
 
 
 def main():

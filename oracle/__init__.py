@@ -135,6 +135,12 @@ def threads_in_use():
     except AttributeError:
         info["sched_affinity"] = None
     try:
+        with open("/sys/fs/cgroup/cpu.max") as f:  # "<quota> <period>" in microseconds, or "max <period>"
+            quota, period = f.read().split()[:2]
+        info["cgroup_cpu_share"] = None if quota == "max" else round(int(quota) / int(period), 2)
+    except (OSError, ValueError):
+        info["cgroup_cpu_share"] = None
+    try:
         info["omp_max_threads"] = int(ctypes.CDLL("libgomp.so.1").omp_get_max_threads())
     except OSError:
         info["omp_max_threads"] = None
