@@ -19,8 +19,11 @@ LIB = os.path.join(HERE, "libcuBERT.so")
 ARCH = "gfx950"
 INCLUDES = ["-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(CSRC, "kernels"), "-I" + os.path.join(CSRC, "host")]
 # -packed-fp32-ops is switched off: hipcc must not form v_pk_*_f32 from scalar float code.
+# -amdgpu-mfma-vgpr-form: matrix-core accumulators stay in ordinary vector registers.  The default puts them in the
+# accumulation registers and copies every result out before the first ordinary instruction can touch it (96 copies
+# per wavefront in the one-launch attention kernel) and, with both files in use, holds fewer wavefronts per SIMD.
 DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
-                "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+                "-packed-fp32-ops", "-mllvm", "-amdgpu-mfma-vgpr-form=1", "-Wno-unused-command-line-argument"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument"]
 
 DEVICE_SOURCES = ["kernels/layernorm.hip", "kernels/softmax.hip", "kernels/elementwise.hip", "kernels/attention.hip", "kernels/gemm_skinny.hip", "kernels/split.hip",

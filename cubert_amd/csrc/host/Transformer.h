@@ -91,11 +91,11 @@ private:
     // out[tokens, out_features] = in[tokens, in_features] * kernel (+ bias) (, GELU); returns whether bias and
     // activation were applied (false: the caller's fused kernel still has to).
     bool dense(int out_features, int tokens, int in_features, const T *kernel, const T *packed, const T *in, T *out,
-               const T *bias, bool bias_in_gemm, bool gelu);
+               const T *bias, bool bias_in_gemm, bool gelu, int ld_out = 0);
     // The same on the fp16 matrix cores from two-term operands (fp32 models only): `in` is split into
     // split_operand first, or, when null, split_operand already holds the [hi | hi | lo] rows.  `bias` may be null.
     void dense_split(int out_features, int tokens, int in_features, const SplitKernel &kernel, const T *in, T *out,
-                     const T *bias);
+                     const T *bias, int ld_out = 0);
 
     void *cublas;
     Profiler *profiler = nullptr;
@@ -111,7 +111,8 @@ private:
     Arena buffers;
     std::vector<Layer> layers;
 
-    T *qkv_out;              // [M, 3*hidden]
+    size_t qkv_ld = 0;       // elements from one token's Q | K | V row to the next (>= 3*hidden)
+    T *qkv_out;              // [M, qkv_ld]
     T *attention_scores;     // [B, heads, seq, seq]
     T *context_out;          // [M, hidden]
     T *attention_output;     // [M, hidden]

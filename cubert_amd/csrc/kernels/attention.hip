@@ -24,6 +24,7 @@
 #include <atomic>
 #include <cstdlib>
 #include <initializer_list>
+#include <string>
 
 #include "cubert_kernels.h"
 #include "device_common.h"
@@ -468,6 +469,250 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
             store_context<T, SPLIT>(ctx, ld_ctx, first_row + acc_row(i, hh), h * D + jt * 32 + r, out[jt][i], split_width,
                                     split_scale);
         }
+    }
+}
+
+// ---- the same for fp16 storage with the ordinary-instruction work cut down ----
+// Counters on attention_fused_kernel<half> at 128 keys showed the vector ALU, not memory or the matrix cores, as its
+// busiest unit: 13 ordinary instructions per score.  This variant computes the same thing with about 5:
+//  * key tiles (32 keys) are classified from the mask row, read as 32-bit words with scalar loads: a tile whose keys
+//    are all masked is left out of the arithmetic altogether when the sequence has an unmasked key -- a
+//    masked key's exp is exactly 0 in fp32 there; a tile whose keys are all kept needs no mask term, so its maximum
+//    is taken over the raw products and scale, change of base and the subtraction of the maximum are one
+//    multiply-add in front of v_exp_f32; only tiles with kept and masked keys (at most one per sequence with a
+//    prefix mask), and every tile of a sequence without any kept key (there the shift cancels, as in the
+//    reference), take the general path of attention_fused_kernel;
+//  * the row sums come out of the matrix cores: the unnormalised probabilities (rounded to fp16, the operand type)
+//    are multiplied with a tile of ones next to V, which leaves every query's sum in the accumulator layout of the
+//    context tiles, where the division by it is 32 multiplications per lane instead of 64 plus 64 additions;
+//  * V is loaded like K, with coalesced 16-byte loads, and kept in LDS as it is in memory ([key][head column]); the
+//    B operand of P V (8 keys of one head column per lane) is transposed on its way out of LDS by two
+//    ds_read_b64_tr_b16 (gfx950): in a group of 16 lanes, lane i names 4 consecutive columns of row i / 4 at column
+//    block i % 4 of a 4 x 16 patch, and lane j receives column j of the patch, rows 0..3.  (The general kernel
+//    gathers V^T from memory with 32 two-byte loads per thread; that gather was measured to cost 6-16 us of 65-77
+//    at 256 sequences x 16 heads x 128 keys.)  Rows of V are pitched so that the four rows of a patch fall on
+//    different banks;
+//  * the context tile leaves through LDS as full 128-byte row segments (4 stores per lane instead of 32 two-byte
+//    ones).
+// Needs the mask (if any) readable as words and ctx rows 16-byte aligned; the launcher falls back otherwise.
+typedef _Float16 v4f16 __attribute__((ext_vector_type(4)));
+
+// ds_read_b64_tr_b16: see the comment above for what arrives in which lane.
+__device__ __forceinline__ v4f16 lds_read_transposed(const half_t *p) {
+    typedef short v4i16 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) v4i16 lds_v4i16;
+    return __builtin_bit_cast(v4f16, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16 *) p));
+}
+
+// Halves per row of V in LDS: the 32 lanes of a lane half read 4 rows x 64 bytes at once, which fall on different
+// banks when the pitch is an odd multiple of 64 bytes (64 banks of 4 bytes).
+template <int D>
+constexpr int fused_half_v_pitch() {
+    return ((D * 2 + 63) / 128 * 128 + 64) / 2;
+}
+
+// LDS bytes of attention_fused_half_kernel<D, KT>: K rows (padded by 16 bytes), V rows, additive mask.
+template <int D, int KT>
+constexpr size_t fused_half_lds_bytes() {
+    constexpr int S = KT * 32;
+    return (size_t) S * (D + 8) * 2 + (size_t) S * fused_half_v_pitch<D>() * 2 + S * sizeof(float);
+}
+
+template <int D, int KT>
+__global__ __launch_bounds__(KT * kWave) void attention_fused_half_kernel(const half_t *__restrict__ q,
+                                                                          const half_t *__restrict__ k,
+                                                                          const half_t *__restrict__ v, int ld,
+                                                                          const int8_t *__restrict__ mask,
+                                                                          half_t *__restrict__ ctx, int ld_ctx,
+                                                                          float alpha, int heads) {
+    typedef half_t T;
+    constexpr int V = 8;
+    constexpr int kSteps = D / 2 / V;
+    constexpr int kColTiles = D / 32;
+    constexpr int S = KT * 32;
+    constexpr int kThreads = KT * kWave;
+    constexpr int kPitchK = D + V;
+    constexpr int kPitchV = fused_half_v_pitch<D>();  // halves per row of V
+    constexpr int kPitchOut = D + V;  // staged context rows: +16 bytes keeps rows 4 apart on different banks
+    constexpr unsigned kAllTiles = (1u << KT) - 1u;
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *s_k = reinterpret_cast<T *>(smem);                 // [S][kPitchK]; later the staged context tiles
+    T *s_v = s_k + S * kPitchK;                           // [S][kPitchV], as in memory
+    float *s_mask = reinterpret_cast<float *>(s_v + S * kPitchV);  // [S] additive mask
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int r = lane & 31, hh = lane >> 5;
+    const int qt = wave_in_block();
+    const int bh = blockIdx.x;
+    const int b = bh / heads, h = bh - b * heads;
+    const T *k_head = k + (size_t) b * S * ld + (size_t) h * D;
+    const T *v_head = v + (size_t) b * S * ld + (size_t) h * D;
+
+    const T *q_row = q + ((size_t) b * S + qt * 32 + r) * ld + (size_t) h * D + hh * (D / 2);
+    Vec<T, V> qv[kSteps];
+#pragma unroll
+    for (int t = 0; t < kSteps; ++t) qv[t] = load_vec<T, V>(q_row + t * V);
+
+    constexpr int kVecPerRow = D / V;
+    constexpr int kLoads = S * kVecPerRow / kThreads;     // = D / V / 2 vectors per thread, for K and for V
+    Vec<T, V> kreg[kLoads], vreg[kLoads];
+    // (every tile is loaded, also those the mask will leave out: with at most 128 keys a workgroup's time is a
+    // chain of latencies, and loads that wait for the mask words would add one more link to it)
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+        const int idx = threadIdx.x + u * kThreads;
+        const int row = idx / kVecPerRow, c = idx - row * kVecPerRow;
+        kreg[u] = load_vec<T, V>(k_head + row * ld + c * V);
+    }
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+        const int idx = threadIdx.x + u * kThreads;
+        const int row = idx / kVecPerRow, c = idx - row * kVecPerRow;
+        vreg[u] = load_vec<T, V>(v_head + row * ld + c * V);
+    }
+
+    // bit kt of keep_any: tile kt has a kept key; of keep_all: all of its keys are kept (workgroup-uniform)
+    unsigned keep_any = kAllTiles, keep_all = kAllTiles;
+    if (mask != nullptr) {
+        const uint32_t *words = reinterpret_cast<const uint32_t *>(mask + (size_t) b * S);
+        keep_any = 0, keep_all = 0;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            uint32_t any = 0, every = 0x80808080u;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t w = words[kt * 8 + i];
+                any |= w;
+                every &= ((w & 0x7f7f7f7fu) + 0x7f7f7f7fu) | w;  // bit 7 of a byte: that byte is not zero
+            }
+            keep_any |= (any != 0 ? 1u : 0u) << kt;
+            keep_all |= ((every & 0x80808080u) == 0x80808080u ? 1u : 0u) << kt;
+        }
+        if (keep_any == 0) keep_any = kAllTiles;  // no kept key at all: every tile, general path
+    }
+    if (!(alpha > 0.f)) keep_all = 0;             // the shortcut takes the maximum before scaling
+    keep_any = __builtin_amdgcn_readfirstlane(keep_any);
+    keep_all = __builtin_amdgcn_readfirstlane(keep_all);
+
+    const bool general_tiles = (keep_any & ~keep_all) != 0;  // uniform
+    if (general_tiles) {
+        for (int i = threadIdx.x; i < S; i += kThreads) {
+            s_mask[i] = !mask[(size_t) b * S + i] ? kMaskedScore * kLog2e : 0.f;  // (mask is not null here)
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+        const int idx = threadIdx.x + u * kThreads;
+        const int row = idx / kVecPerRow, c = idx - row * kVecPerRow;
+        store_vec<T, V>(s_k + row * kPitchK + c * V, kreg[u]);
+    }
+    __syncthreads();  // K and the mask are in LDS; the V loads are still in flight
+
+    // scores^T[key, query], in p[kt]: raw products for an all-kept tile, log2-unit masked scores for a general one
+    const float scale = alpha * kLog2e;
+    v16f32 p[KT];
+    float mx = -3.402823466e+38f;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        v16f32 c = {};
+        if ((keep_any >> kt) & 1u) {
+#pragma unroll
+            for (int t = 0; t < kSteps; ++t) {
+                Mma<T>::run(c, load_vec<T, V>(s_k + (kt * 32 + r) * kPitchK + hh * (D / 2) + t * V), qv[t]);
+            }
+            if ((keep_all >> kt) & 1u) {
+                float raw = c[0];
+#pragma unroll
+                for (int i = 1; i < 16; ++i) raw = fmaxf(raw, c[i]);
+                mx = fmaxf(mx, raw * scale);
+            } else {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const Vec<float, 4> m = load_vec<float, 4>(s_mask + kt * 32 + g * 8 + hh * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float sc = fmaf(c[g * 4 + e], scale, m.v[e]);
+                        c[g * 4 + e] = sc;
+                        mx = fmaxf(mx, sc);
+                    }
+                }
+            }
+        }
+        p[kt] = c;
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float shift = -mx;
+
+    // V goes to LDS only now: its loads had the whole score phase to arrive
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+        const int idx = threadIdx.x + u * kThreads;
+        const int row = idx / kVecPerRow, c = idx - row * kVecPerRow;
+        store_vec<T, V>(s_v + row * kPitchV + c * V, vreg[u]);
+    }
+    __syncthreads();  // (also: every wavefront is done with K, whose space the context tiles use below)
+
+    // ctx[query, column] and, in `total`, every query's sum of probabilities: A slots = this lane's unnormalised
+    // probabilities, B = the same keys of column jt*32 + r of V, or ones.  The lane's slots of step (kt, run) are
+    // keys kt*32 + run*16 + hh*4 + {0..3} and the same + 8: one transposing read each.  In its group of 16 lanes
+    // (group g: columns (g & 1) * 16 .. + 15, lane half g >> 1), lane i names row i / 4 and column block i % 4.
+    const int tr_group = lane >> 4, tr_i = lane & 15;
+    const T *tr_base = s_v + ((tr_group >> 1) * 4 + (tr_i >> 2)) * kPitchV + (tr_group & 1) * 16 + (tr_i & 3) * 4;
+    v16f32 out[kColTiles], total = {};
+#pragma unroll
+    for (int jt = 0; jt < kColTiles; ++jt) out[jt] = v16f32{};
+    Vec<T, V> ones;
+#pragma unroll
+    for (int e = 0; e < V; ++e) ones.v[e] = (T) 1.f;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        if (!((keep_any >> kt) & 1u)) continue;
+        const bool fast = (keep_all >> kt) & 1u;
+#pragma unroll
+        for (int run = 0; run < 16 / V; ++run) {
+            Vec<T, V> a;
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+                const float x = p[kt][run * V + e];
+                a.v[e] = from_f32<T>(__builtin_amdgcn_exp2f(fast ? fmaf(x, scale, shift) : x + shift));
+            }
+#pragma unroll
+            for (int jt = 0; jt < kColTiles; ++jt) {
+                const T *at = tr_base + (kt * 32 + run * 16) * kPitchV + jt * 32;
+                Vec<T, V> bv;
+                const v4f16 lo = lds_read_transposed(at), hi = lds_read_transposed(at + 8 * kPitchV);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    bv.v[e] = lo[e];
+                    bv.v[4 + e] = hi[e];
+                }
+                Mma<T>::run(out[jt], a, bv);
+            }
+            Mma<T>::run(total, a, ones);
+        }
+    }
+
+    // lane holds output column jt*32 + r of 16 query rows and, in total[i], the sum of row acc_row(i, hh)
+    T *stage = s_k + qt * 32 * kPitchOut;  // this wavefront's 32 x D tile
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const float inv = __builtin_amdgcn_rcpf(total[i]);
+#pragma unroll
+        for (int jt = 0; jt < kColTiles; ++jt) {
+            stage[acc_row(i, hh) * kPitchOut + jt * 32 + r] = from_f32<T>(out[jt][i] * inv);
+        }
+    }
+    // the same wavefront reads back what it staged; LDS operations of one wavefront complete in order
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    __builtin_amdgcn_wave_barrier();
+    constexpr int kChunks = D / V;             // 16-byte chunks per row
+    constexpr int kRowsPerPass = kWave / kChunks;
+    const int chunk = lane % kChunks, row_in = lane / kChunks;
+    T *dst = ctx + ((size_t) b * S + qt * 32) * ld_ctx + (size_t) h * D + chunk * V;
+#pragma unroll
+    for (int pass = 0; pass < 32 / kRowsPerPass; ++pass) {
+        const int row = row_in + kRowsPerPass * pass;
+        store_vec<T, V>(dst + row * ld_ctx, load_vec<T, V>(stage + row * kPitchOut + chunk * V));
     }
 }
 
@@ -1143,6 +1388,27 @@ int launch_fused_kt(const T *q, const T *k, const T *v, int ld, const int8_t *ma
         }
     }
     if (split_width > 0) return CUBERT_UNSUPPORTED;
+    if constexpr (sizeof(T) == 2) {
+        // CUBERT_ATTENTION_KERNEL=general / lean in the environment forces one of the two; by default the lean kernel
+        // runs where the grid fills the chip several times over (measured at 128 keys, head size 64: 4096 workgroups
+        // 65.6 -> 57.0 us) and the general one where a workgroup's own chain of latencies is what takes the time
+        // (384 workgroups: 10.8 us against 11.3 with the lean kernel's extra pass through LDS on the way out).
+        static const int forced = [] {
+            const char *e = getenv("CUBERT_ATTENTION_KERNEL");
+            return e == nullptr ? 0 : (std::string(e) == "general" ? 1 : (std::string(e) == "lean" ? 2 : 0));
+        }();
+        const bool lean = forced == 2 || (forced == 0 && batch * heads >= 1024);
+        if (lean && (mask == nullptr || is_aligned(mask, 4)) && is_aligned(ctx, 16) && ld_ctx % 8 == 0) {
+            auto kernel = attention_fused_half_kernel<D, KT>;
+            constexpr size_t half_lds = fused_half_lds_bytes<D, KT>();
+            if (half_lds > 48 * 1024) {
+                static std::atomic<unsigned long long> raised{0};  // per instantiation
+                if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
+            }
+            return launch_untimed(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) half_lds, s, q, k, v, ld,
+                                  mask, ctx, ld_ctx, alpha, heads);
+        }
+    }
     auto kernel = attention_fused_kernel<T, D, KT, false>;
     if (lds > 48 * 1024) {
         static std::atomic<unsigned long long> raised{0};  // per instantiation

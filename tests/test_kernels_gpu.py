@@ -568,6 +568,53 @@ def test_attention_fused_against_oracle(K, name, batch, heads, seq, d, masked):
     assert_close(host(ctx)[:seq], host(c3)[:seq], 2e-3, "fused vs three kernels %s, fully masked sequence" % name)
 
 
+@pytest.mark.parametrize("batch,heads,seq,d", [(64, 16, 128, 64), (128, 8, 32, 64), (86, 12, 64, 32), (70, 16, 96, 128)])
+@pytest.mark.parametrize("masked", [True, False])
+def test_attention_fused_many_problems_fp16(K, batch, heads, seq, d, masked):
+    """From 1024 (batch, head) problems up, fp16 sequences of at most 128 keys take the kernel that classifies key
+    tiles from the mask words (left out / no mask term / general), takes the row sums from the matrix cores and
+    reads V through transposing LDS loads.  Masks with every tile class: prefixes that end inside a tile and on a
+    tile boundary, kept keys scattered over dead tiles, bytes other than 1, no masked key, one kept key in the last
+    tile, a sequence with no kept key -- against the oracle, which computes every key."""
+    name = "f16"
+    rng = np.random.default_rng(batch + heads * 100 + seq + d)
+    H = heads * d
+    qkv = q(rng.normal(0, 1, (batch * seq, 3 * H)), name)
+    qh, kh, vh = (np.ascontiguousarray(x) for x in (qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:]))
+    valid = rng.integers(1, seq + 1, batch)
+    mask = (np.arange(seq)[None, :] < valid[:, None]).astype(np.int8)
+    mask[0, :] = 0                                      # no kept key: every tile, general path
+    mask[1, :] = 1                                      # every key kept
+    mask[2, :] = 0
+    mask[2, seq - 1] = 1                                # one kept key, in the last tile
+    mask[3, :] = (rng.random(seq) < 0.5).astype(np.int8)
+    mask[3, :32] = 0                                    # a dead tile in front of mixed ones
+    mask[4, :32] = 1                                    # prefix that ends on a tile boundary
+    mask[4, 32:] = 0
+    mask[5, :] = rng.integers(1, 4, seq).astype(np.int8) * (rng.random(seq) < 0.8)   # any non-zero byte keeps the key
+    mask[6, :] = -1                                     # negative bytes keep it too
+    alpha = 1.0 / math.sqrt(d)
+    ctx = K.attention_fused(dev(qkv, tdt(name)), dev(mask) if masked else None, batch, heads, seq, d, alpha)
+    assert ctx is not None
+    scores = oracle.round_to_half(oracle.att_q_k(qh, kh, batch, seq, heads, d, alpha=alpha))
+    if masked:
+        scores = scores + (-10000.0 * (mask == 0).astype(np.float32))[:, None, None, :]
+    p = oracle.softmax_(np.ascontiguousarray(scores.reshape(-1, seq), dtype=np.float32)).reshape(scores.shape)
+    want = oracle.att_qk_v(np.ascontiguousarray(oracle.round_to_half(p), dtype=np.float32), vh, batch, seq, heads,
+                           d).reshape(batch * seq, H)
+    got = host(ctx)
+    for b in range(batch):
+        rows = slice(b * seq, (b + 1) * seq)
+        assert_close(got[rows], want[rows], 2e-3, "attention, many problems, sequence %d (valid %d)" % (b, valid[b]))
+    # the same call on a mask that cannot be read as 32-bit words takes the general kernel: same result to rounding
+    if masked:
+        shifted = torch.zeros(batch * seq + 1, dtype=torch.int8, device="cuda")
+        shifted[1:] = dev(mask).reshape(-1)
+        general = K.attention_fused(dev(qkv, tdt(name)), shifted[1:].reshape(batch, seq), batch, heads, seq, d, alpha)
+        assert general is not None
+        assert_close(got, host(general), 2e-3, "tile-classifying kernel vs general kernel")
+
+
 @pytest.mark.parametrize("name", ["f32", "f16"])
 @pytest.mark.parametrize("heads,seq,d", [(2, 512, 64), (3, 256, 64), (2, 160, 64), (1, 384, 32), (2, 512, 32)])
 def test_attention_long_sequences_with_padding(K, name, heads, seq, d):
