@@ -1422,8 +1422,9 @@ template <typename T, int D>
 int launch_fused(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
                  int batch, int heads, int seq, int split_width, float split_scale, hipStream_t s) {
     if constexpr (D == 64) {
-        // fewer problems than compute units: split each over four wavefronts (5.3 -> 3.x us at 12 heads)
-        if (seq == 32 && batch * heads <= 256 && (mask == nullptr || is_aligned(mask, 4))) {
+        // split each problem over four wavefronts: a quarter of the dependent matrix instructions per wavefront
+        // (12 problems 5.3 -> 4.7 us, 1536 problems 15.95 -> 15.0 us; not measured beyond)
+        if (seq == 32 && batch * heads <= 2048 && (mask == nullptr || is_aligned(mask, 4))) {
             if constexpr (sizeof(T) == 4) {
                 if (split_width > 0) {
                     return launch_untimed(attention_small_kernel<T, true>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q,

@@ -520,9 +520,9 @@ def test_attention_scores_and_context(K, name, batch, heads, seq, d):
 @pytest.mark.parametrize("name", ["f32", "f16"])
 @pytest.mark.parametrize("batch,heads,seq,d", [(3, 12, 32, 64), (2, 4, 128, 64), (2, 3, 64, 32), (1, 2, 96, 128),
                                                (2, 16, 128, 64), (5, 1, 32, 64), (7, 3, 64, 64),
-                                               # seq 32, head size 64: four wavefronts per problem up to 256
-                                               # problems (above), one wavefront per problem beyond (below)
-                                               (1, 12, 32, 64), (24, 12, 32, 64), (2, 2, 32, 32),
+                                               # seq 32, head size 64: four wavefronts per problem up to 2048
+                                               # problems, one wavefront per problem beyond and at head size 32
+                                               (1, 12, 32, 64), (24, 12, 32, 64), (180, 12, 32, 64), (2, 2, 32, 32),
                                                # longer than 128: the online-softmax kernels (chunks of 64 keys;
                                                # seq 512 stages the keys in groups, the others the whole head)
                                                (1, 2, 512, 64), (2, 3, 256, 64), (2, 2, 160, 64), (1, 1, 384, 32),
