@@ -161,10 +161,12 @@ void Transformer<T>::layout_weights() {
 template <typename T>
 void Transformer<T>::layout_buffers() {
     const size_t M = max_batch_size * seq_length, H = hidden_size;
-    // Rows packed without padding.  (64 elements of padding per row take the one-launch attention kernel from 57 to
-    // 51 us at 256 sequences x 16 heads x 128 keys, fp16 -- a row pitch of 6 KB spreads badly over the memory
-    // channels -- but the forward pass as a whole was 1.2 % slower with it, 20.75 against 20.51 ms.)
-    qkv_ld = 3 * H;
+    // 64 elements between one token's Q | K | V row and the next: the attention kernels read 128-byte pieces of these
+    // rows at the row pitch, and a pitch of 3 * hidden elements (6 KB for BERT-large in fp16) spreads those pieces
+    // badly over the memory channels.  Measured at 256 sequences x 16 heads x 128 keys, fp16, with and without the
+    // padding in alternation on one box: attention kernel 57.4 -> 51.3 us, forward pass 20.34 -> 20.24 ms; BERT-base
+    // shapes (pitch 4.5 KB fp16, 9 KB fp32) move by less than the run-to-run noise.
+    qkv_ld = 3 * H + 64;
     qkv_out = buffers.take<T>(M * qkv_ld);
     attention_scores = buffers.take<T>(max_batch_size * num_attention_heads * seq_length * seq_length);
     context_out = buffers.take<T>(M * H);
