@@ -612,20 +612,25 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_half_kernel(const 
     const float scale = alpha * kLog2e;
     v16f32 p[KT];
     float mx = -3.402823466e+38f;
+    // (The empty asm statements keep the workgroup-uniform tests below as branches: folded into selects, both sides
+    // of each would be computed for every score.)
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
-        v16f32 c = {};
         if ((keep_any >> kt) & 1u) {
+            asm volatile("");
+            v16f32 c = {};
 #pragma unroll
             for (int t = 0; t < kSteps; ++t) {
                 Mma<T>::run(c, load_vec<T, V>(s_k + (kt * 32 + r) * kPitchK + hh * (D / 2) + t * V), qv[t]);
             }
             if ((keep_all >> kt) & 1u) {
+                asm volatile("");
                 float raw = c[0];
 #pragma unroll
                 for (int i = 1; i < 16; ++i) raw = fmaxf(raw, c[i]);
                 mx = fmaxf(mx, raw * scale);
             } else {
+                asm volatile("");
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const Vec<float, 4> m = load_vec<float, 4>(s_mask + kt * 32 + g * 8 + hh * 4);
@@ -637,8 +642,8 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_half_kernel(const 
                     }
                 }
             }
+            p[kt] = c;
         }
-        p[kt] = c;
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
     const float shift = -mx;
@@ -667,15 +672,21 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_half_kernel(const 
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
         if (!((keep_any >> kt) & 1u)) continue;
-        const bool fast = (keep_all >> kt) & 1u;
+        asm volatile("");
+        Vec<T, V> a[16 / V];
+        if ((keep_all >> kt) & 1u) {
+            asm volatile("");
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                a[i / V].v[i % V] = from_f32<T>(__builtin_amdgcn_exp2f(fmaf(p[kt][i], scale, shift)));
+            }
+        } else {
+            asm volatile("");
+#pragma unroll
+            for (int i = 0; i < 16; ++i) a[i / V].v[i % V] = from_f32<T>(__builtin_amdgcn_exp2f(p[kt][i] + shift));
+        }
 #pragma unroll
         for (int run = 0; run < 16 / V; ++run) {
-            Vec<T, V> a;
-#pragma unroll
-            for (int e = 0; e < V; ++e) {
-                const float x = p[kt][run * V + e];
-                a.v[e] = from_f32<T>(__builtin_amdgcn_exp2f(fast ? fmaf(x, scale, shift) : x + shift));
-            }
 #pragma unroll
             for (int jt = 0; jt < kColTiles; ++jt) {
                 const T *at = tr_base + (kt * 32 + run * 16) * kPitchV + jt * 32;
@@ -686,9 +697,9 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_half_kernel(const 
                     bv.v[e] = lo[e];
                     bv.v[4 + e] = hi[e];
                 }
-                Mma<T>::run(out[jt], a, bv);
+                Mma<T>::run(out[jt], a[run], bv);
             }
-            Mma<T>::run(total, a, ones);
+            Mma<T>::run(total, a[run], ones);
         }
     }
 
