@@ -92,6 +92,9 @@ SIGNATURES = {
     "cubert_event_record": (ci, [vp, vp]),
     "cubert_event_elapsed_ms": (ci, [vp, vp, ctypes.POINTER(cf)]),
     "cubert_time_next_launch": (ci, [vp, vp]),
+    "cubert_attention_order": (ci, [vp, ci, ci, vp, vp]),
+    "cubert_attention_fused_ordered_f32": (ci, [vp, vp, vp, ci, vp, vp, vp, ci, cf, ci, ci, ci, ci, vp]),
+    "cubert_attention_fused_ordered_f16": (ci, [vp, vp, vp, ci, vp, vp, vp, ci, cf, ci, ci, ci, ci, vp]),
     "cubert_gemm_skinny_noalloc_f32": (ci, [vp, ci, ci, ci, cf, vp, ci, vp, ci, vp, ci, vp, ci]),
     "cubert_gemm_skinny_packed_elements": (ctypes.c_size_t, [ci, ci]),
     "cubert_gemm_f16_f32": (ci, [vp, ci, ci, ci, ci, ci, cf, vp, ci, vp, ci, cf, vp, ci, vp]),

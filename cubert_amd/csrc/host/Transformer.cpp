@@ -170,6 +170,7 @@ void Transformer<T>::layout_buffers() {
     qkv_out = buffers.take<T>(M * qkv_ld);
     attention_scores = buffers.take<T>(max_batch_size * num_attention_heads * seq_length * seq_length);
     context_out = buffers.take<T>(M * H);
+    attention_order = buffers.take<int>(max_batch_size);
     attention_output = buffers.take<T>(M * H);
     intermediate_output = buffers.take<T>(M * intermediate_size);
     layer_output[0] = buffers.take<T>(M * H);
@@ -217,7 +218,10 @@ bool Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *ma
                 return true;
             }
         }
-        if (cuBERT::attention_fused(Q, K, V, ld, mask, context_out, H, alpha, B, A, S, d, stream)) return false;
+        if (cuBERT::attention_fused(Q, K, V, ld, mask, context_out, H, alpha, B, A, S, d, stream,
+                                    order_ready ? attention_order : nullptr)) {
+            return false;
+        }
         fused_attention_fits = false;  // seq_length and head size are fixed per model: do not ask again
     }
 
@@ -309,6 +313,10 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
     // in fp32: they keep the fp32 kernels)
     const bool split = split_dense && (size_t) M >= kTwoTermMinTokens;
     bool operand_ready = false;
+
+    // long sequences: the attention kernels take the sequences longest first (the mask is the same for every layer)
+    order_ready = seq_length > 128 && attention_mask != nullptr && fused_attention_fits &&
+                  cuBERT::attention_order(attention_mask, (int) batch_size, (int) seq_length, attention_order, stream);
 
     T *prev_output = input_gpu;
     for (size_t l = 0; l < num_hidden_layers; ++l) {

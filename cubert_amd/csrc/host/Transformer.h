@@ -115,6 +115,8 @@ private:
     T *qkv_out;              // [M, qkv_ld]
     T *attention_scores;     // [B, heads, seq, seq]
     T *context_out;          // [M, hidden]
+    int *attention_order = nullptr;  // [max_batch]: sequence indices, most live key tiles first (seq_length > 128)
+    bool order_ready = false;        // attention_order holds the current request's order
     T *attention_output;     // [M, hidden]
     T *intermediate_output;  // [M, intermediate]
     T *layer_output[2];      // [M, hidden], alternating between layers

@@ -271,20 +271,31 @@ inline bool attention_context(const half *probs, const half *v, int ld, half *ct
     return true;
 }
 
+// Sequence indices by falling number of live key tiles, for the long-sequence attention kernels; false when the
+// shape or the mask's alignment is not taken (then pass no order).
+inline bool attention_order(const int8_t *mask, int batch, int seq, int *order, void *stream) {
+    const int rc = cubert_attention_order(mask, batch, seq, order, stream);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+
 // The whole attention core (scores, mask, softmax, context) in one launch (seq_length <= 512); false when
 // the shape has no such kernel (reference: AttentionSelf.cpp:96-111 runs it as three operators).
 inline bool attention_fused(const float *q, const float *k, const float *v, int ld, const int8_t *mask, float *ctx,
-                            int ld_ctx, float alpha, int batch, int heads, int seq, int head_size, void *stream) {
-    const int rc = cubert_attention_fused_f32(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, head_size,
-                                              stream);
+                            int ld_ctx, float alpha, int batch, int heads, int seq, int head_size, void *stream,
+                            const int *order = nullptr) {
+    const int rc = cubert_attention_fused_ordered_f32(q, k, v, ld, mask, order, ctx, ld_ctx, alpha, batch, heads, seq,
+                                                      head_size, stream);
     if (rc == CUBERT_UNSUPPORTED) return false;
     CUBERT_CHECK(rc);
     return true;
 }
 inline bool attention_fused(const half *q, const half *k, const half *v, int ld, const int8_t *mask, half *ctx,
-                            int ld_ctx, float alpha, int batch, int heads, int seq, int head_size, void *stream) {
-    const int rc = cubert_attention_fused_f16(h(q), h(k), h(v), ld, mask, h(ctx), ld_ctx, alpha, batch, heads, seq,
-                                              head_size, stream);
+                            int ld_ctx, float alpha, int batch, int heads, int seq, int head_size, void *stream,
+                            const int *order = nullptr) {
+    const int rc = cubert_attention_fused_ordered_f16(h(q), h(k), h(v), ld, mask, order, h(ctx), ld_ctx, alpha, batch,
+                                                      heads, seq, head_size, stream);
     if (rc == CUBERT_UNSUPPORTED) return false;
     CUBERT_CHECK(rc);
     return true;

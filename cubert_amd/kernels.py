@@ -89,11 +89,32 @@ def attention_scores(qkv, batch, heads, seq, head_size, alpha):
     return scores
 
 
-def attention_fused(qkv, mask, batch, heads, seq, head_size, alpha):
-    """ctx[B*S, H] = softmax(alpha Q K^T + mask) V in one launch (seq <= 512); None when the shape does not fit."""
+def attention_order(mask):
+    """Sequence indices by falling number of key tiles (32 keys) with a kept key, as an int32 tensor; None when the
+    shape or the mask's alignment is not taken."""
+    batch, seq = mask.shape
+    order = torch.empty(batch, dtype=torch.int32, device=mask.device)
+    rc = lib().cubert_attention_order(_ptr(mask), batch, seq, _ptr(order), _stream())
+    if rc == -2:
+        return None
+    _check(rc, "cubert_attention_order")
+    return order
+
+
+def attention_fused(qkv, mask, batch, heads, seq, head_size, alpha, order=None):
+    """ctx[B*S, H] = softmax(alpha Q K^T + mask) V in one launch (seq <= 512); None when the shape does not fit.
+    `order` (from attention_order): the sequence each group of `heads` workgroups takes."""
     hidden = heads * head_size
     flat = qkv.view(-1)
     ctx = torch.empty((batch * seq, hidden), dtype=qkv.dtype, device=qkv.device)
+    if order is not None:
+        fn = getattr(lib(), "cubert_attention_fused_ordered_" + _suffix(qkv))
+        rc = fn(_ptr(flat), _ptr(flat[hidden:]), _ptr(flat[2 * hidden:]), 3 * hidden, _ptr(mask), _ptr(order), _ptr(ctx),
+                hidden, float(alpha), batch, heads, seq, head_size, _stream())
+        if rc == -2:
+            return None
+        _check(rc, fn.__name__)
+        return ctx
     fn = getattr(lib(), "cubert_attention_fused_" + _suffix(qkv))
     rc = fn(_ptr(flat), _ptr(flat[hidden:]), _ptr(flat[2 * hidden:]), 3 * hidden, _ptr(mask), _ptr(ctx), hidden,
             float(alpha), batch, heads, seq, head_size, _stream())

@@ -126,6 +126,24 @@ int cubert_attention_fused_f16(const cubert_half *q, const cubert_half *k, const
                                const int8_t *mask, cubert_half *ctx, int ld_ctx, float alpha, int batch, int heads,
                                int seq_length, int head_size, void *stream);
 
+/* Longest sequences first.  The long-sequence kernels (seq_length > 128) leave out key tiles (32 keys) whose mask
+ * bytes are all zero, so a workgroup's time goes with its sequence's number of live tiles, and workgroups are handed
+ * to the compute units in index order: a long sequence late in the batch starts late and the launch waits for it.
+ * cubert_attention_order writes the sequence indices 0..batch-1 by falling live-tile count into order[batch] (one
+ * small launch; the mask is the same for every layer of a forward pass, so once per pass);
+ * cubert_attention_fused_ordered_* is cubert_attention_fused_* taking sequence order[i] where it would take i
+ * (order may be NULL: batch order; shapes of at most 128 keys ignore it).  Results are identical with any order.
+ * CUBERT_UNSUPPORTED from cubert_attention_order (seq_length not a multiple of 32 or above 512, more than 4096
+ * sequences, a mask that is not 4-byte aligned): pass NULL.
+ * No counterpart in the reference, which computes every key of every sequence (src/cuBERT/op_att/AttentionSelf.cpp:96-111). */
+int cubert_attention_order(const int8_t *mask, int batch, int seq_length, int *order, void *stream);
+int cubert_attention_fused_ordered_f32(const float *q, const float *k, const float *v, int ld, const int8_t *mask,
+                                       const int *order, float *ctx, int ld_ctx, float alpha, int batch, int heads,
+                                       int seq_length, int head_size, void *stream);
+int cubert_attention_fused_ordered_f16(const cubert_half *q, const cubert_half *k, const cubert_half *v, int ld,
+                                       const int8_t *mask, const int *order, cubert_half *ctx, int ld_ctx, float alpha,
+                                       int batch, int heads, int seq_length, int head_size, void *stream);
+
 
 /* Row softmax of a [rows, channel] matrix, in place or not (classifier probabilities).
  * replaces: softmax_<T>(in, out, rows, channel, sum_buf, stream), reference src/cuBERT/op/Softmax.h:8-14. */

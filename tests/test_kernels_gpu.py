@@ -665,6 +665,42 @@ def test_attention_long_sequences_with_padding(K, name, heads, seq, d):
     assert_close(got[keep], host(plain)[keep], 1e-6 if name == "f32" else 2e-3, "skipping vs not skipping, tight")
 
 
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("batch,heads,seq,d", [(37, 3, 512, 64), (9, 2, 256, 64), (5, 2, 160, 32)])
+def test_attention_longest_sequences_first(K, name, batch, heads, seq, d):
+    """cubert_attention_order sorts the sequences by falling number of live key tiles (a sequence without any kept
+    key counts as full); the long-sequence kernels give bit for bit the same context whichever order they are handed."""
+    rng = np.random.default_rng(batch + seq)
+    H = heads * d
+    if name == "f32" and seq != 512 and seq * (d + 4) * 4 + d * (seq + 4) * 4 + 2 * seq * 4 > 160 * 1024:
+        pytest.skip("K and V of one head do not fit the LDS in fp32")
+    valid = np.minimum(seq, 1 + np.floor(rng.exponential(seq / 5.0, batch))).astype(np.int64)
+    mask = (np.arange(seq)[None, :] < valid[:, None]).astype(np.int8)
+    mask[1, :] = 0                                     # no kept key: every tile is computed
+    mask[2, :] = 0
+    mask[2, seq - 3] = 1                               # a single live tile, the last one
+    mask[3, ::37] = 1                                  # kept keys scattered over every tile
+    dmask = dev(mask)
+    order = K.attention_order(dmask)
+    assert order is not None
+    got = order.cpu().numpy().astype(np.int64)
+    assert sorted(got.tolist()) == list(range(batch))
+    live = (mask.reshape(batch, seq // 32, 32) != 0).any(-1).sum(-1)
+    live[live == 0] = seq // 32
+    assert (np.diff(live[got]) <= 0).all(), live[got]
+    qkv = dev(q(rng.normal(0, 1, (batch * seq, 3 * H)), name), tdt(name))
+    alpha = 1.0 / math.sqrt(d)
+    plain = K.attention_fused(qkv, dmask, batch, heads, seq, d, alpha)
+    ordered = K.attention_fused(qkv, dmask, batch, heads, seq, d, alpha, order=order)
+    backwards = K.attention_fused(qkv, dmask, batch, heads, seq, d, alpha, order=order.flip(0).contiguous())
+    assert plain is not None and ordered is not None and backwards is not None
+    assert torch.equal(plain, ordered) and torch.equal(plain, backwards)
+    # shapes and masks the sort declines
+    assert K.attention_order(dev(np.ones((3, 40), np.int8))) is None
+    odd = torch.zeros(batch * seq + 1, dtype=torch.int8, device="cuda")[1:].reshape(batch, seq)
+    assert K.attention_order(odd) is None
+
+
 def test_attention_unsupported_shapes_are_declined(K):
     """Shapes without a matrix-core kernel return CUBERT_UNSUPPORTED and launch nothing; the host classes then
     loop the strided-batched GEMM (covered by the encoder reference vectors, seq 4, head size 3)."""
