@@ -39,33 +39,46 @@ TRAFFIC_PROFILE = "profiles/traffic_pmc.md"
 TRAFFIC_SOURCE = {  # kernel kind -> (source file under cubert_amd/csrc/kernels, first 16 hex digits of its SHA-256)
     "bias_gelu": ("elementwise.hip", "59dcc33f61344079"),
     "bias_tanh": ("elementwise.hip", "59dcc33f61344079"),
-    "bias_res_ln": ("layernorm.hip", "3fc1f92646a53b40"),
-    "embed_ln": ("layernorm.hip", "3fc1f92646a53b40"),
+    "bias_res_ln": ("layernorm.hip", "4c00fd91a55914b9"),
+    "embed_ln": ("layernorm.hip", "4c00fd91a55914b9"),
     "mask_scale_softmax": ("softmax.hip", "90a529eac55169fa"),
-    "attention_fused": ("attention.hip", "ca1212b0708528de"),
+    "mean_pool": ("elementwise.hip", "59dcc33f61344079"),
+    "classifier_head": ("elementwise.hip", "59dcc33f61344079"),
+    "attention_fused": ("attention.hip", "61ce7581b6d55693"),
 }
 MEASURED_TRAFFIC = {
     "C1": {
-        "attention_fused": 50675000,
-        "embed_ln": 25286438,
-        "mask_scale_softmax": 12588575,
-        "bias_res_ln": 37627533,
-        "bias_gelu": 100321862
+        "embed_ln": 25318226,
+        "attention_fused": 50105055,
+        "bias_res_ln": 37617779,
+        "bias_gelu": 100340735,
+        "classifier_head": 934243,
+        "mask_scale_softmax": 12589813
+    },
+    "C2": {
+        "embed_ln": 12906152,
+        "attention_fused": 25138599,
+        "bias_res_ln": 18866016,
+        "bias_gelu": 50185077,
+        "mean_pool": 6324901,
+        "classifier_head": 147215,
+        "mask_scale_softmax": 25117523
     },
     "C3": {
-        "attention_fused": 124900000,
-        "embed_ln": 99683567,
-        "mask_scale_softmax": 801872210,
-        "bias_res_ln": 150175758,
-        "bias_gelu": 400874437
+        "embed_ln": 99781532,
+        "attention_fused": 130332429,
+        "bias_res_ln": 150207744,
+        "bias_gelu": 400909955,
+        "classifier_head": 308663,
+        "mask_scale_softmax": 801926025
     },
     "C4": {
-        "attention_fused": 266970000,
-        "embed_ln": 133391970,
-        "mask_scale_softmax": 267485530,
-        "bias_res_ln": 200172741,
-        "bias_gelu": 534484085,
-        "bias_tanh": 1110678
+        "embed_ln": 133791775,
+        "attention_fused": 267267723,
+        "bias_res_ln": 200205373,
+        "bias_gelu": 534519097,
+        "classifier_head": 1199487,
+        "mask_scale_softmax": 267503783
     }
 }
 
