@@ -243,7 +243,7 @@ def cpu_baseline(workload, cfg, w, ids, mask, seg):
         gomp = None
     wf = {k: oracle.round_to_half(v) for k, v in w.items()} if half else w
     vars_obj = oracle.Vars(wf)
-    n = min(cfg["batch"], 128)  # bounded sample: at most 128 sequences of the workload per pass
+    n = min(cfg["batch"], 128, max(1, 8192 // S))  # bounded sample: at most 128 sequences and 8192 tokens per pass
 
     def leg(threads, max_passes, budget_s):
         oracle.set_blas_threads(threads)

@@ -175,6 +175,7 @@ int build_plan(BlasContext *ctx, const GemmKey &k, GemmPlan *plan) {
 
 constexpr double kTuneMinFlops = 1e9;
 constexpr int kTuneRuns = 8;
+constexpr int kTunePasses = 2;
 constexpr float kTuneMinGain = 0.97f;  // leave the heuristic's first choice unless another is at least 3 % faster
 
 bool tuning_enabled() {
@@ -216,29 +217,44 @@ void tune_plan(BlasContext *ctx, const GemmKey &k, GemmPlan &p, float alpha, con
         }
     }
     const float beta = 0.f;
+    // Two passes over the candidates, each candidate judged by the faster of its two bursts: the chip's clocks move
+    // while the timing runs, and a candidate timed once during a slow spell would lose to a worse one.
+    std::vector<float> fastest(p.candidates.size(), 0.f);
+    for (int pass = 0; pass < kTunePasses; ++pass) {
+        for (int i = 0; i < (int) p.candidates.size(); ++i) {
+            if (pass > 0 && fastest[i] == 0.f) continue;  // failed in the first pass
+            hipblasLtMatmulAlgo_t *algo = &p.candidates[i].algo;
+            bool ok = true;
+            if (pass == 0) {  // warm-up, also a check
+                ok = hipblasLtMatmul(ctx->lt, p.desc, &alpha, A, p.a, B, p.b, &beta, C, p.c, C, p.c, algo, ctx->workspace,
+                                     kWorkspaceBytes, ctx->stream) == HIPBLAS_STATUS_SUCCESS;
+                if (!ok) continue;
+            }
+            if (hipEventRecord(ctx->tune_start, ctx->stream) != hipSuccess) return;
+            for (int r = 0; r < kTuneRuns && ok; ++r) {
+                ok = hipblasLtMatmul(ctx->lt, p.desc, &alpha, A, p.a, B, p.b, &beta, C, p.c, C, p.c, algo, ctx->workspace,
+                                     kWorkspaceBytes, ctx->stream) == HIPBLAS_STATUS_SUCCESS;
+            }
+            float ms = 0.f;
+            if (hipEventRecord(ctx->tune_stop, ctx->stream) != hipSuccess ||
+                hipEventSynchronize(ctx->tune_stop) != hipSuccess ||
+                hipEventElapsedTime(&ms, ctx->tune_start, ctx->tune_stop) != hipSuccess) {
+                (void) hipGetLastError();
+                return;
+            }
+            if (!ok) {
+                fastest[i] = 0.f;
+                continue;
+            }
+            if (fastest[i] == 0.f || ms < fastest[i]) fastest[i] = ms;
+        }
+    }
     int best = 0;
-    float best_ms = 0.f, first_ms = 0.f;
+    float best_ms = 0.f;
+    const float first_ms = fastest[0];
     for (int i = 0; i < (int) p.candidates.size(); ++i) {
-        hipblasLtMatmulAlgo_t *algo = &p.candidates[i].algo;
-        bool ok = hipblasLtMatmul(ctx->lt, p.desc, &alpha, A, p.a, B, p.b, &beta, C, p.c, C, p.c, algo, ctx->workspace,
-                                  kWorkspaceBytes, ctx->stream) == HIPBLAS_STATUS_SUCCESS;  // warm-up, also a check
-        if (!ok) continue;
-        if (hipEventRecord(ctx->tune_start, ctx->stream) != hipSuccess) return;
-        for (int r = 0; r < kTuneRuns && ok; ++r) {
-            ok = hipblasLtMatmul(ctx->lt, p.desc, &alpha, A, p.a, B, p.b, &beta, C, p.c, C, p.c, algo, ctx->workspace,
-                                 kWorkspaceBytes, ctx->stream) == HIPBLAS_STATUS_SUCCESS;
-        }
-        float ms = 0.f;
-        if (hipEventRecord(ctx->tune_stop, ctx->stream) != hipSuccess ||
-            hipEventSynchronize(ctx->tune_stop) != hipSuccess ||
-            hipEventElapsedTime(&ms, ctx->tune_start, ctx->tune_stop) != hipSuccess) {
-            (void) hipGetLastError();
-            return;
-        }
-        if (!ok) continue;
-        if (i == 0) first_ms = ms;
-        if (best_ms == 0.f || ms < best_ms) {
-            best_ms = ms;
+        if (fastest[i] > 0.f && (best_ms == 0.f || fastest[i] < best_ms)) {
+            best_ms = fastest[i];
             best = i;
         }
     }
