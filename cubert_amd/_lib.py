@@ -128,6 +128,7 @@ for _t in ("f32", "f16"):
         "cubert_gemm_skinny_pack_" + _t: (ci, [vp, vp, ci, ci, ci, vp]),
         "cubert_gemm_skinny_packed_" + _t: (ci, [vp, ci, ci, ci, cf, vp, vp, ci, vp, ci, vp, ci]),
         "cubert_gemm_strided_batch_" + _t: (ci, [vp, ci, ci, ci, ci, ci, cf, vp, ci, cll, vp, ci, cll, cf, vp, ci, cll, ci]),
+        "cubert_gemm_batch_" + _t: (ci, [vp, ci, ci, ci, ci, ci, cf, vp, ci, vp, ci, cf, vp, ci, ci]),
     })
 
 

@@ -26,7 +26,7 @@ DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-Xclang
                 "-packed-fp32-ops", "-mllvm", "-amdgpu-mfma-vgpr-form=1", "-Wno-unused-command-line-argument"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument"]
 
-DEVICE_SOURCES = ["kernels/layernorm.hip", "kernels/softmax.hip", "kernels/elementwise.hip", "kernels/attention.hip", "kernels/gemm_skinny.hip", "kernels/split.hip",
+DEVICE_SOURCES = ["kernels/layernorm.hip", "kernels/softmax.hip", "kernels/elementwise.hip", "kernels/attention.hip", "kernels/gemm_skinny.hip", "kernels/gemm_batch.hip", "kernels/split.hip",
                   "runtime.hip"]
 HOST_SOURCES = ["host/Transformer.cpp", "host/Bert.cpp", "host/BertM.cpp", "host/Graph.cpp", "host/tokenization.cpp",
                 "host/api.cpp"]

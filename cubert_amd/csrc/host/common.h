@@ -164,6 +164,22 @@ inline void blas_gemm_strided_batch(void *handle, bool TransA, bool TransB, int 
                                                strideB, beta, h(C), ldc, strideC, batchCount));
 }
 
+// reference: common.h:70-80 (arrays of device pointers, themselves in device memory)
+inline void blas_gemm_batch(void *handle, bool TransA, bool TransB, int m, int n, int k, float alpha,
+                            const float **Aarray, int lda, const float **Barray, int ldb, float beta, float **Carray,
+                            int ldc, int batchCount) {
+    CUBERT_CHECK(cubert_gemm_batch_f32(handle, TransA, TransB, m, n, k, alpha, Aarray, lda, Barray, ldb, beta, Carray,
+                                       ldc, batchCount));
+}
+inline void blas_gemm_batch(void *handle, bool TransA, bool TransB, int m, int n, int k, float alpha,
+                            const half **Aarray, int lda, const half **Barray, int ldb, float beta, half **Carray,
+                            int ldc, int batchCount) {
+    CUBERT_CHECK(cubert_gemm_batch_f16(handle, TransA, TransB, m, n, k, alpha,
+                                       reinterpret_cast<const cubert_half *const *>(Aarray), lda,
+                                       reinterpret_cast<const cubert_half *const *>(Barray), ldb, beta,
+                                       reinterpret_cast<cubert_half *const *>(Carray), ldc, batchCount));
+}
+
 // ---- layer launchers (names of the reference's launchers where one exists) ----
 
 // reference: op/Embedding.h:9-15

@@ -32,6 +32,10 @@ int gemm_skinny_noalloc_f32(int M, int N, int K, float alpha, const float *A, in
                             int ldc, const float *bias, int activation, hipStream_t stream);
 template <typename T>
 int gemm_skinny_pack(const T *A, int lda, int M, int K, T *packed, hipStream_t stream);
+// kernels/gemm_batch.hip
+template <typename T>
+int gemm_batch(int transA, int transB, int M, int N, int K, float alpha, const T *const *A_array, int lda,
+               const T *const *B_array, int ldb, float beta, T *const *C_array, int ldc, int batch, hipStream_t stream);
 
 LaunchTiming &pending_launch_timing() {
     static thread_local LaunchTiming pending;
@@ -654,6 +658,29 @@ int cubert_gemm_strided_batch_f16(void *handle, int transA, int transB, int M, i
                                   int batch_count) {
     return run_gemm(handle, 1, transA, transB, M, N, K, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC,
                     batch_count, nullptr);
+}
+
+int cubert_gemm_batch_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha,
+                          const float *const *A_array, int lda, const float *const *B_array, int ldb, float beta,
+                          float *const *C_array, int ldc, int batch_count) {
+    BlasContext *ctx = (BlasContext *) handle;
+    if (!ctx) return CUBERT_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    ctx->used = true;
+    return cubert::gemm_batch<float>(transA, transB, M, N, K, alpha, A_array, lda, B_array, ldb, beta, C_array, ldc,
+                                     batch_count, ctx->stream);
+}
+
+int cubert_gemm_batch_f16(void *handle, int transA, int transB, int M, int N, int K, float alpha,
+                          const cubert_half *const *A_array, int lda, const cubert_half *const *B_array, int ldb,
+                          float beta, cubert_half *const *C_array, int ldc, int batch_count) {
+    BlasContext *ctx = (BlasContext *) handle;
+    if (!ctx) return CUBERT_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    ctx->used = true;
+    return cubert::gemm_batch<cubert::half_t>(transA, transB, M, N, K, alpha, (const cubert::half_t *const *) A_array,
+                                              lda, (const cubert::half_t *const *) B_array, ldb, beta,
+                                              (cubert::half_t *const *) C_array, ldc, batch_count, ctx->stream);
 }
 
 }  // extern "C"

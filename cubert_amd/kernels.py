@@ -285,3 +285,14 @@ class Blas(object):
         _call("cubert_gemm_strided_batch", C, self.handle, int(transA), int(transB), M, N, K, float(alpha), _ptr(A),
               lda, sA, _ptr(B), ldb, sB, float(beta), _ptr(C), ldc, sC, batch)
         return C
+
+    def gemm_batch(self, transA, transB, M, N, K, alpha, As, lda, Bs, ldb, beta, Cs, ldc):
+        """One problem per entry of As / Bs / Cs (lists of tensors, which may be views into larger buffers): the
+        entry point takes device arrays of device pointers, built here (reference: blas_gemm_batch)."""
+        def pointers(ts):
+            return torch.tensor([t.data_ptr() for t in ts], dtype=torch.int64).cuda()
+        pa, pb, pc = pointers(As), pointers(Bs), pointers(Cs)
+        _call("cubert_gemm_batch", Cs[0], self.handle, int(transA), int(transB), M, N, K, float(alpha), _ptr(pa), lda,
+              _ptr(pb), ldb, float(beta), _ptr(pc), ldc, len(Cs))
+        self._keep = (pa, pb, pc)  # the launch is asynchronous: the pointer arrays must outlive it
+        return Cs

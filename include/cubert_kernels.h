@@ -338,6 +338,20 @@ int cubert_gemm_strided_batch_f16(void *handle, int transA, int transB, int M, i
                                   int ldb, long long strideB, float beta, cubert_half *C, int ldc,
                                   long long strideC, int batch_count);
 
+/* The same over `batch_count` problems given as arrays of pointers: A_array, B_array and C_array are DEVICE arrays
+ * of batch_count device pointers (one problem each, as cublasGemmBatchedEx takes them); lda, ldb, ldc and the
+ * transposes are shared.  fp32 accumulation; with beta = 0 the C matrices are not read.  Runs on the handle's
+ * stream, asynchronously.  This is the interface of the reference's attention contractions (Att_Q_K / Att_QK_V
+ * build one pointer per (batch, head), src/cuBERT/op_att/BatchMatMul.cpp:31-38,57-68,103-110,129-140); the host
+ * classes here use cubert_attention_* instead, which is the fast path.
+ * replaces: blas_gemm_batch<T>, reference src/cuBERT/common.h:70-80 (src/cuBERT/common.cpp:261-298,375-396). */
+int cubert_gemm_batch_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha,
+                          const float *const *A_array, int lda, const float *const *B_array, int ldb, float beta,
+                          float *const *C_array, int ldc, int batch_count);
+int cubert_gemm_batch_f16(void *handle, int transA, int transB, int M, int N, int K, float alpha,
+                          const cubert_half *const *A_array, int lda, const cubert_half *const *B_array, int ldb,
+                          float beta, cubert_half *const *C_array, int ldc, int batch_count);
+
 #ifdef __cplusplus
 }
 #endif

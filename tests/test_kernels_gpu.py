@@ -171,6 +171,58 @@ def test_batch_matmul_reference_vectors(K, case):
     np.testing.assert_array_equal(host(out).reshape(B, S, A, d), want)
 
 
+def test_batch_matmul_reference_vectors_pointer_arrays(K, case):
+    """The same vectors through blas_gemm_batch's interface, called as the reference's Att_Q_K / Att_QK_V call it
+    (src/cuBERT/op_att/BatchMatMul.cpp:31-38,57-68,103-110,129-140): one pointer per (batch, head) into the
+    [B, S, A, d] operands, scores laid out [B, S_q, A, S_k] as in the reference."""
+    blas = K.Blas()
+    S, A, d, B = 2, 4, 3, 2
+    H = A * d
+    c = case(T + "op_att/BatchMatMulTest.cpp", "q_k")
+    q_, k_ = dev(np.array(c.arrays["query"], np.float32)), dev(np.array(c.arrays["key"], np.float32))
+    out = torch.full((B * S * A * S,), 7.0, device="cuda")
+    problems = [(b, h) for b in range(B) for h in range(A)]
+    idx = lambda b, h: b * S * d * A + d * h
+    blas.gemm_batch(True, False, S, S, d, 1.0, [k_[idx(b, h):] for b, h in problems], H,
+                    [q_[idx(b, h):] for b, h in problems], H, 0.0,
+                    [out[b * S * S * A + S * h:] for b, h in problems], S * A)
+    c.check(host(out))
+    c = case(T + "op_att/BatchMatMulTest.cpp", "qk_v")
+    p_, v_ = dev(np.array(c.arrays["qk"], np.float32)), dev(np.array(c.arrays["value"], np.float32))
+    out = torch.full((B * S * H,), 7.0, device="cuda")
+    blas.gemm_batch(False, False, d, S, S, 1.0, [v_[idx(b, h):] for b, h in problems], H,
+                    [p_[b * S * S * A + S * h:] for b, h in problems], S * A, 0.0,
+                    [out[idx(b, h):] for b, h in problems], H)
+    c.check(host(out))
+
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
+@pytest.mark.parametrize("M,N,K_,batch", [(32, 32, 64, 24), (64, 128, 128, 5), (70, 65, 19, 3), (1, 1, 1, 2),
+                                          (128, 128, 64, 7), (5, 200, 33, 4)])
+def test_gemm_batch_against_oracle_sgemm(K, name, ta, tb, M, N, K_, batch):
+    """blas_gemm_batch (arrays of pointers, column-major, all transposes, alpha / beta, padded leading dimensions,
+    tile edges) against the oracle's sgemm problem by problem."""
+    rng = np.random.default_rng(M * 31 + N * 7 + K_ + batch + 2 * ta + tb)
+    lda, ldb, ldc = (K_ if ta else M) + 3, (N if tb else K_) + 2, M + 1
+    a_cols, b_cols = (M if ta else K_), (K_ if tb else N)
+    As = [q(rng.normal(0, 1, lda * a_cols), name) for _ in range(batch)]
+    Bs = [q(rng.normal(0, 1, ldb * b_cols), name) for _ in range(batch)]
+    C0 = [q(rng.normal(0, 1, ldc * N), name) for _ in range(batch)]
+    blas = K.Blas()
+    dA, dB = [dev(a, tdt(name)) for a in As], [dev(b, tdt(name)) for b in Bs]
+    for alpha, beta in ((1.0, 0.0), (0.5, 1.0), (1.0, -0.25)):
+        dC = [dev(c0, tdt(name)) for c0 in C0]
+        blas.gemm_batch(ta, tb, M, N, K_, alpha, dA, lda, dB, ldb, beta, dC, ldc)
+        for z in range(batch):
+            want = oracle.sgemm(ta, tb, M, N, K_, alpha, As[z], lda, Bs[z], ldb, beta, C0[z].copy(), ldc)
+            got = host(dC[z])
+            live = (np.arange(ldc * N) % ldc) < M  # the padding rows of C are not written
+            np.testing.assert_array_equal(got[~live], C0[z][~live])
+            assert_close(got[live], want[live], 2e-5 if name == "f32" else 2e-3,
+                         "gemm_batch %s problem %d alpha=%g beta=%g" % (name, z, alpha, beta))
+
+
 # ------------------------------------------------------------------ seeded parity with the oracle
 
 @pytest.mark.parametrize("name", ["f32", "f16"])
