@@ -265,6 +265,7 @@ void Bert<T>::forward(size_t batch_size) {
             return;
         }
         classifier_head_fits = false;  // the sizes are fixed per model: do not ask again
+        t.cancel();
     }
     if (tanh_pending) {
         Timed t(&profiler, Profiler::kBiasTanh, stream);

@@ -45,11 +45,10 @@ public:
 
     bool on(Kind k) const { return (mask >> k) & 1u; }
 
-    // The layer kernels (kinds 0..6) are one launch each: the launch itself carries the event pair and
-    // the elapsed time is the kernel's execution time.  GEMM kinds may be several library launches, so
-    // they are bracketed by marker events (which adds the gaps between launches), and so is the fused
-    // attention kernel.
-    static bool single_launch(Kind k) { return k < kDenseGemm; }
+    // The layer kernels (kinds 0..6) and the one-launch attention kernel are one launch each: the launch itself
+    // carries the event pair and the elapsed time is the kernel's execution time.  GEMM kinds may be several
+    // library launches, so they are bracketed by marker events (which adds the gaps between launches).
+    static bool single_launch(Kind k) { return k < kDenseGemm || k == kAttentionFused || k == kClassifierHead; }
 
     void begin(Kind k, void *stream) {
         if (!on(k)) return;
@@ -61,8 +60,19 @@ public:
         }
     }
 
+    // The entry point under a single-launch bracket declined and launched nothing: the pair goes back unused.
+    void cancel(Kind k) {
+        if (!on(k) || !single_launch(k)) return;
+        CUBERT_CHECK(cubert_time_next_launch(nullptr, nullptr));
+        cancelled = true;
+    }
+
     void end(Kind k, void *stream) {
         if (!on(k)) return;
+        if (cancelled) {
+            cancelled = false;
+            return;
+        }
         if (!single_launch(k)) CUBERT_CHECK(cubert_event_record(pool[used].second, stream));
         kinds_used.push_back(k);
         ++used;
@@ -94,6 +104,7 @@ private:
     }
 
     unsigned mask = 0;
+    bool cancelled = false;
     size_t used = 0;
     std::vector<std::pair<void *, void *>> pool;
     std::vector<Kind> kinds_used;
@@ -107,6 +118,10 @@ public:
     }
     ~Timed() {
         if (p) p->end(k, stream);
+    }
+    // nothing was launched inside this bracket
+    void cancel() {
+        if (p) p->cancel(k);
     }
 
 private:

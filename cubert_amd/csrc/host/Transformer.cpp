@@ -223,6 +223,7 @@ bool Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *ma
             return false;
         }
         fused_attention_fits = false;  // seq_length and head size are fixed per model: do not ask again
+        t.cancel();
     }
 
     const bool loop_heads = A <= B;

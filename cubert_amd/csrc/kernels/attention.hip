@@ -1447,7 +1447,7 @@ int launch_fused_kt(const T *q, const T *k, const T *v, int ld, const int8_t *ma
                 static std::atomic<unsigned long long> raised{0};  // per instantiation
                 if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
             }
-            return launch_untimed(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask,
+            return launch_lds(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask,
                                   ctx, ld_ctx, alpha, heads, split_width, split_scale);
         }
     }
@@ -1469,7 +1469,7 @@ int launch_fused_kt(const T *q, const T *k, const T *v, int ld, const int8_t *ma
                 static std::atomic<unsigned long long> raised{0};  // per instantiation
                 if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
             }
-            return launch_untimed(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) half_lds, s, q, k, v, ld,
+            return launch_lds(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) half_lds, s, q, k, v, ld,
                                   mask, ctx, ld_ctx, alpha, heads);
         }
     }
@@ -1478,7 +1478,7 @@ int launch_fused_kt(const T *q, const T *k, const T *v, int ld, const int8_t *ma
         static std::atomic<unsigned long long> raised{0};  // per instantiation
         if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
     }
-    return launch_untimed(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask, ctx,
+    return launch_lds(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask, ctx,
                           ld_ctx, alpha, heads, split_width, split_scale);
 }
 
@@ -1491,12 +1491,12 @@ int launch_fused(const T *q, const T *k, const T *v, int ld, const int8_t *mask,
         if (seq == 32 && batch * heads <= 2048 && (mask == nullptr || is_aligned(mask, 4))) {
             if constexpr (sizeof(T) == 4) {
                 if (split_width > 0) {
-                    return launch_untimed(attention_small_kernel<T, true>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q,
+                    return launch_lds(attention_small_kernel<T, true>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q,
                                           k, v, ld, mask, ctx, ld_ctx, alpha, heads, split_width, split_scale);
                 }
             }
             if (split_width > 0) return CUBERT_UNSUPPORTED;
-            return launch_untimed(attention_small_kernel<T, false>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q, k, v,
+            return launch_lds(attention_small_kernel<T, false>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q, k, v,
                                   ld, mask, ctx, ld_ctx, alpha, heads, split_width, split_scale);
         }
     }
@@ -1532,13 +1532,13 @@ int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask,
                                    ((size_t) seq + 16 * 32) * sizeof(float);
         if constexpr (sizeof(T) == 4) {
             if (split_width > 0) {
-                return launch_untimed(attention_flash_grouped_kernel<T, D, true>, dim3(batch * heads), dim3(1024),
+                return launch_lds(attention_flash_grouped_kernel<T, D, true>, dim3(batch * heads), dim3(1024),
                                       (unsigned) grouped_lds, s, q, k, v, ld, mask, ctx, ld_ctx, alpha, heads,
                                       skip_masked_tiles, split_width, split_scale, order);
             }
         }
         if (split_width > 0) return CUBERT_UNSUPPORTED;
-        return launch_untimed(attention_flash_grouped_kernel<T, D, false>, dim3(batch * heads), dim3(1024),
+        return launch_lds(attention_flash_grouped_kernel<T, D, false>, dim3(batch * heads), dim3(1024),
                               (unsigned) grouped_lds, s, q, k, v, ld, mask, ctx, ld_ctx, alpha, heads, skip_masked_tiles,
                               split_width, split_scale, order);
     }
@@ -1548,7 +1548,7 @@ int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask,
             auto kernel = attention_flash_kernel<T, D, true>;
             static std::atomic<unsigned long long> raised{0};  // per instantiation
             if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
-            return launch_untimed(kernel, dim3(batch * heads), dim3(seq / 32 * kWave), (unsigned) lds, s, q, k, v, ld,
+            return launch_lds(kernel, dim3(batch * heads), dim3(seq / 32 * kWave), (unsigned) lds, s, q, k, v, ld,
                                   mask, ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles, split_width, split_scale, order);
         }
     }
@@ -1556,7 +1556,7 @@ int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask,
     auto kernel = attention_flash_kernel<T, D, false>;
     static std::atomic<unsigned long long> raised{0};  // per instantiation
     if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
-    return launch_untimed(kernel, dim3(batch * heads), dim3(seq / 32 * kWave), (unsigned) lds, s, q, k, v, ld, mask,
+    return launch_lds(kernel, dim3(batch * heads), dim3(seq / 32 * kWave), (unsigned) lds, s, q, k, v, ld, mask,
                           ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles, split_width, split_scale, order);
 }
 
