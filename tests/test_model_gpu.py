@@ -166,6 +166,53 @@ CONFIG_CASES = [
 ]
 
 
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_randomly_drawn_model_configurations(cb, seed):
+    """Fifteen models per seed with every size drawn at random -- heads, head size (also ones no matrix-core kernel
+    takes), seq_length (1 ... 512, not only multiples of 32), intermediate size, layers, labels (few and many), with and
+    without pooler / classifier / classifier bias, both compute types, prefix and scattered masks, a batch below the
+    maximum -- against the oracle, every output; two calls in a row must agree bit for bit.  The fp32 bound here is
+    5e-5, not 1e-5: weights are drawn with a standard deviation of 0.05 instead of 0.02, and on such a model the
+    oracle itself is up to 1e-5 away from a float64 evaluation (summation order over 1536 ... 3080 terms), so two fp32
+    evaluations are up to 3e-5 apart (measured over 480 drawn models: 2.8e-5; fp16: 1.3e-2)."""
+    from cubert_amd.testing import random_bert_weights, random_inputs
+    rng = np.random.default_rng(seed)
+    for case in range(15):
+        heads = int(rng.choice([1, 2, 3, 4, 8, 12]))
+        d = int(rng.choice([32, 64, 64, 64, 128, 16, 24]))
+        hidden = heads * d
+        seq = int(rng.choice([1, 4, 7, 32, 32, 64, 96, 128, 160, 256, 512, 33]))
+        if seq * hidden > 512 * 512:
+            seq = 32
+        max_batch = int(rng.integers(1, 9))
+        batch = int(rng.integers(1, max_batch + 1))
+        layers = int(rng.integers(1, 4))
+        inter = int(rng.choice([hidden * 4, hidden * 2 + 8, 100, 3 * hidden]))
+        labels = int(rng.choice([1, 2, 3, 7, 70]))
+        pooler, classifier, cbias = bool(rng.integers(0, 2)), bool(rng.integers(0, 4) > 0), bool(rng.integers(0, 2))
+        compute_type = int(rng.integers(0, 2))
+        vocab = int(rng.integers(5, 400))
+        scattered = bool(rng.integers(0, 2))
+        what = "seed %d case %d: B=%d/%d S=%d H=%d A=%d I=%d L=%d labels=%d pooler=%s classifier=%s bias=%s %s %s" % (
+            seed, case, batch, max_batch, seq, hidden, heads, inter, layers, labels, pooler, classifier, cbias,
+            "f16" if compute_type else "f32", "scattered" if scattered else "prefix")
+        print(what, flush=True)
+        w = random_bert_weights(seed=seed * 100 + case, vocab=vocab, hidden=hidden, layers=layers, heads=heads,
+                                intermediate=inter, max_position=max(seq, 8), type_vocab=2, labels=labels, pooler=pooler,
+                                classifier=classifier, classifier_bias=cbias, ln_random=True, stddev=0.05)
+        ids, mask, seg = random_inputs(seed=seed * 100 + case, batch=batch, seq_length=seq, vocab=vocab,
+                                       min_valid=None if scattered else 1, max_valid=None if scattered else seq,
+                                       segment_split="random" if seq > 1 else None, scattered_mask=scattered)
+        bert = cb.Bert(w, max_batch, seq, layers, heads, compute_type=compute_type)
+        got, again = bert.forward(ids, mask, seg), bert.forward(ids, mask, seg)
+        bert.close()
+        seen = {k: (oracle.round_to_half(v) if compute_type else v) for k, v in w.items()}
+        want = oracle.bert_forward(seen, ids, mask, seg, layers, heads)
+        for k, ref in want.items():
+            assert np.array_equal(got[k], again[k]), what + ": " + k + " differs between two calls"
+            assert_close(got[k], ref, 5e-5 if compute_type == 0 else 2 * FP16_TOL, what + ": " + k)
+
+
 @pytest.mark.parametrize("name,rows", CONFIG_CASES)
 def test_benchmark_configurations(cb, name, rows):
     """The five workloads at their real shapes (BERT-base / BERT-large, random-init N(0, 0.02))."""
