@@ -309,12 +309,13 @@ __global__ __launch_bounds__(kBlock) void attention_context_kernel(const T *__re
 constexpr float kMaskedScore = -10000.0f;
 constexpr float kLog2e = 1.4426950408889634f;
 
+// A probability from its exponential: times the reciprocal of the row's sum (one division per query instead of one
+// per score; at 128 sequences x 12 heads x 32 keys in fp32 the divisions were 0.7 us of a 12.4 us launch).  Within
+// 1.5 units in the last place of the quotient the reference forms (src/cuBERT/op/Softmax.cpp:32-35).
 template <typename T>
-__device__ __forceinline__ float normalise_prob(float e, float sum, float inv_sum);
-template <>
-__device__ __forceinline__ float normalise_prob<float>(float e, float sum, float) { return e / sum; }
-template <>
-__device__ __forceinline__ float normalise_prob<half_t>(float e, float, float inv_sum) { return e * inv_sum; }
+__device__ __forceinline__ float normalise_prob(float e, float, float inv_sum) {
+    return e * inv_sum;
+}
 
 // LDS bytes of attention_fused_kernel<T, D, KT>: K rows, V^T rows (both padded by 16 bytes), additive mask.
 template <typename T, int D, int KT>
