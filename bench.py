@@ -44,41 +44,41 @@ TRAFFIC_SOURCE = {  # kernel kind -> (source file under cubert_amd/csrc/kernels,
     "mask_scale_softmax": ("softmax.hip", "90a529eac55169fa"),
     "mean_pool": ("elementwise.hip", "59dcc33f61344079"),
     "classifier_head": ("elementwise.hip", "59dcc33f61344079"),
-    "attention_fused": ("attention.hip", "61ce7581b6d55693"),
+    "attention_fused": ("attention.hip", "fd800e8d4c9ccee9"),
 }
 MEASURED_TRAFFIC = {
     "C1": {
-        "embed_ln": 25318226,
-        "attention_fused": 50105055,
-        "bias_res_ln": 37617779,
-        "bias_gelu": 100340735,
+        "embed_ln": 25318195,
+        "attention_fused": 50098109,
+        "bias_res_ln": 37618237,
+        "bias_gelu": 100340642,
         "classifier_head": 934243,
-        "mask_scale_softmax": 12589813
+        "mask_scale_softmax": 12589795
     },
     "C2": {
-        "embed_ln": 12906152,
-        "attention_fused": 25138599,
-        "bias_res_ln": 18866016,
-        "bias_gelu": 50185077,
-        "mean_pool": 6324901,
+        "embed_ln": 12906209,
+        "attention_fused": 25138580,
+        "bias_res_ln": 18866004,
+        "bias_gelu": 50185062,
+        "mean_pool": 6324895,
         "classifier_head": 147215,
-        "mask_scale_softmax": 25117523
+        "mask_scale_softmax": 25117455
     },
     "C3": {
-        "embed_ln": 99781532,
-        "attention_fused": 130332429,
-        "bias_res_ln": 150207744,
-        "bias_gelu": 400909955,
+        "embed_ln": 99789147,
+        "attention_fused": 130327065,
+        "bias_res_ln": 150209246,
+        "bias_gelu": 400910315,
         "classifier_head": 308663,
-        "mask_scale_softmax": 801926025
+        "mask_scale_softmax": 801925601
     },
     "C4": {
-        "embed_ln": 133791775,
-        "attention_fused": 267267723,
-        "bias_res_ln": 200205373,
-        "bias_gelu": 534519097,
+        "embed_ln": 133804718,
+        "attention_fused": 267259400,
+        "bias_res_ln": 200205923,
+        "bias_gelu": 534518836,
         "classifier_head": 1199487,
-        "mask_scale_softmax": 267503783
+        "mask_scale_softmax": 267503616
     }
 }
 
