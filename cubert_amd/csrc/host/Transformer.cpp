@@ -168,7 +168,6 @@ void Transformer<T>::layout_buffers() {
     // shapes (pitch 4.5 KB fp16, 9 KB fp32) move by less than the run-to-run noise.
     qkv_ld = 3 * H + 64;
     qkv_out = buffers.take<T>(M * qkv_ld);
-    attention_scores = buffers.take<T>(max_batch_size * num_attention_heads * seq_length * seq_length);
     context_out = buffers.take<T>(M * H);
     attention_order = buffers.take<int>(max_batch_size);
     attention_output = buffers.take<T>(M * H);
@@ -176,6 +175,17 @@ void Transformer<T>::layout_buffers() {
     layer_output[0] = buffers.take<T>(M * H);
     layer_output[1] = buffers.take<T>(M * H);
     if (split_dense) split_operand = buffers.take<half>(M * 3 * (H > intermediate_size ? H : intermediate_size));
+}
+
+template <typename T>
+T *Transformer<T>::scores() {
+    if (attention_scores == nullptr) {
+        const size_t count = max_batch_size * num_attention_heads * seq_length * seq_length;
+        score_memory.take<T>(count);
+        score_memory.allocate();
+        attention_scores = score_memory.take<T>(count);
+    }
+    return attention_scores;
 }
 
 template <typename T>
@@ -226,6 +236,7 @@ bool Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *ma
         t.cancel();
     }
 
+    T *score_tensor = scores();
     const bool loop_heads = A <= B;
     const int outer = loop_heads ? A : B, inner = loop_heads ? B : A;
     const long long in_outer = loop_heads ? head_stride : seq_stride, in_inner = loop_heads ? seq_stride : head_stride;
@@ -235,25 +246,25 @@ bool Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *ma
 
     {
         Timed t(profiler, Profiler::kAttentionGemm, stream);
-        if (!cuBERT::attention_scores(Q, K, ld, attention_scores, alpha, B, A, S, d, stream)) {
+        if (!cuBERT::attention_scores(Q, K, ld, score_tensor, alpha, B, A, S, d, stream)) {
             for (int o = 0; o < outer; ++o) {
                 // column-major: scores_ba (S_k x S_q, ld S) = K_ba^T (d x S_k, ld 3H)^T * Q_ba (d x S_q, ld 3H)
                 cuBERT::blas_gemm_strided_batch(cublas, true, false, S, S, d, alpha, K + o * in_outer, ld, in_inner,
-                                                Q + o * in_outer, ld, in_inner, 0.f, attention_scores + o * sc_outer,
+                                                Q + o * in_outer, ld, in_inner, 0.f, score_tensor + o * sc_outer,
                                                 S, sc_inner, inner);
             }
         }
     }
     {
         Timed t(profiler, Profiler::kMaskScaleSoftmax, stream);
-        cuBERT::mask_scale_softmax_(attention_scores, mask, 1.0f, B, A, S, stream);
+        cuBERT::mask_scale_softmax_(score_tensor, mask, 1.0f, B, A, S, stream);
     }
     Timed t(profiler, Profiler::kAttentionGemm, stream);
-    if (!cuBERT::attention_context(attention_scores, V, ld, context_out, H, B, A, S, d, stream)) {
+    if (!cuBERT::attention_context(score_tensor, V, ld, context_out, H, B, A, S, d, stream)) {
         for (int o = 0; o < outer; ++o) {
             // column-major: ctx_ba (d x S_q, ld H) = V_ba (d x S_k, ld 3H) * p_ba (S_k x S_q, ld S)
             cuBERT::blas_gemm_strided_batch(cublas, false, false, d, S, S, 1.f, V + o * in_outer, ld, in_inner,
-                                            attention_scores + o * sc_outer, S, sc_inner, 0.f,
+                                            score_tensor + o * sc_outer, S, sc_inner, 0.f,
                                             context_out + o * ctx_outer, H, ctx_inner, inner);
         }
     }

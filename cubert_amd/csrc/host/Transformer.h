@@ -85,6 +85,10 @@ private:
 
     void layout_weights();
     void layout_buffers();
+    // The [max_batch, heads, seq, seq] score tensor.  Only the three-kernel attention path touches it, and the
+    // one-launch kernel takes every BERT shape up to seq_length 512, so it is not part of `buffers` (it would be the
+    // largest of them: 403 MB at batch 64 x 12 heads x seq 512 in fp16) but allocated on first use.
+    T *scores();
     // context_out = attention(qkv); with `split_context` (fp32 models in the two-term Dense form) the one-launch
     // kernel writes the context there as two-term rows instead and true is returned
     bool attention(size_t batch_size, const T *qkv, const int8_t *mask, half *split_context = nullptr);
@@ -109,11 +113,12 @@ private:
 
     Arena weights;
     Arena buffers;
+    Arena score_memory;  // the score tensor of the three-kernel attention path: claimed when a request first takes it
     std::vector<Layer> layers;
 
     size_t qkv_ld = 0;       // elements from one token's Q | K | V row to the next (>= 3*hidden)
     T *qkv_out;              // [M, qkv_ld]
-    T *attention_scores;     // [B, heads, seq, seq]
+    T *attention_scores = nullptr;  // [B, heads, seq, seq], in score_memory (null until scores() is first called)
     T *context_out;          // [M, hidden]
     int *attention_order = nullptr;  // [max_batch]: sequence indices, most live key tiles first (seq_length > 128)
     bool order_ready = false;        // attention_order holds the current request's order
