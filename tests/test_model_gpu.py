@@ -317,6 +317,37 @@ def test_sequences_of_a_batch_are_independent_at_full_size(cb):
         assert_close(alone[k], first[k][3:4], 2e-3, "single sequence, " + k)
 
 
+@pytest.mark.parametrize("name", ["C1", "C3"])
+def test_masked_positions_reach_no_kept_position_at_full_size(cb, name):
+    """A size-independent property of the mask at benchmark shapes (C1: fp32, 128 x 32, prefix masks; C3: fp16, 64 x 512,
+    heavy padding, where the attention kernel leaves out key tiles without a kept key): a masked key sits 10000 below
+    every kept one, its exponential is exactly 0 in fp32, so what the tokens at masked positions are -- ids and segment
+    ids -- cannot change a single bit at any kept position, nor in the BertPooler's output, the logits or the
+    probabilities (all from position 0, which is kept).  The outputs at the masked positions themselves do change."""
+    from cubert_amd.testing import CONFIGS, config_inputs, config_weights
+    cfg = CONFIGS[name]
+    m = cfg["model"]
+    batch = min(cfg["batch"], 32)
+    w = config_weights(name, seed=0)
+    ids, mask, seg = config_inputs(name, seed=0, batch=batch)
+    assert mask[:, 0].all() and not mask.all()
+    rng = np.random.default_rng(17)
+    other_ids = np.where(mask != 0, ids, rng.integers(0, m["vocab"], ids.shape, dtype=np.int32)).astype(np.int32)
+    other_seg = np.where(mask != 0, seg, 1 - seg).astype(np.int8)
+    bert = cb.Bert(w, batch, cfg["seq_length"], m["layers"], m["heads"], 0 if cfg["dtype"] == "f32" else 1)
+    first = bert.forward(ids, mask, seg, to_float=False)
+    second = bert.forward(other_ids, mask, other_seg, to_float=False)
+    bert.close()
+    kept = mask != 0
+    for k in ("logits", "probs"):
+        assert np.array_equal(first[k], second[k]), k
+    if cfg["pooler"]:
+        assert np.array_equal(first["pooled_output"], second["pooled_output"])
+    for k in ("sequence_output", "embedding_output"):
+        assert np.array_equal(first[k][kept], second[k][kept]), k + " at kept positions"
+    assert not np.array_equal(first["embedding_output"][~kept], second["embedding_output"][~kept])
+
+
 # ------------------------------------------------------------------ the public C API on a GraphDef file
 
 @pytest.fixture(scope="module")
