@@ -79,6 +79,7 @@ SIGNATURES = {
     "cubert_gpu_info": (ci, [ci]),
     "cubert_malloc": (vp, [ctypes.c_size_t]),
     "cubert_free": (ci, [vp]),
+    "cubert_mem_info": (ci, [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]),
     "cubert_memcpy": (ci, [vp, vp, ctypes.c_size_t, ci]),
     "cubert_memcpy_async": (ci, [vp, vp, ctypes.c_size_t, ci, vp]),
     "cubert_stream_create": (vp, []),

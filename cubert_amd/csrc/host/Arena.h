@@ -26,11 +26,12 @@ public:
         return base_ == nullptr ? nullptr : reinterpret_cast<U *>(base_ + offset);
     }
 
-    // Ends the measuring pass: allocates what was asked for and rewinds.
+    // Ends the measuring pass: allocates what was asked for and rewinds.  When the allocation fails (cuBERT::malloc
+    // throws) the arena is empty and measuring again, so a later attempt asks for the same amount, not for more.
     void allocate() {
         size_ = cursor_;
-        base_ = static_cast<char *>(cuBERT::malloc(size_ == 0 ? kAlign : size_));
         cursor_ = 0;
+        base_ = static_cast<char *>(cuBERT::malloc(size_ == 0 ? kAlign : size_));
     }
 
     bool measuring() const { return base_ == nullptr; }

@@ -216,6 +216,11 @@ Graph<T>::Graph(const char *filename) {
         if (content_len == 0 && listed > 0) {
             const size_t declared = declared_elements(value.dims);
             len = declared >= listed && declared <= kMaxExpandedElements ? declared : listed;
+        } else if (content_len == 0 && !value.dims.empty()) {
+            // neither bytes nor a value list, but a declared shape: how TensorFlow's tensor compression writes a
+            // tensor whose elements are all zero (proto3 drops the default value of the one listed element)
+            const size_t declared = declared_elements(value.dims);
+            if (declared <= kMaxExpandedElements) len = declared;
         }
 
         storage.emplace_back(new T[len]);
@@ -233,13 +238,13 @@ Graph<T>::Graph(const char *filename) {
             }
         } else if (len > 0) {
             if (value.dtype == kDtFloat) {
-                std::vector<float> tmp(len, value.float_val.back());
+                std::vector<float> tmp(len, listed > 0 ? value.float_val.back() : 0.f);
                 std::copy(value.float_val.begin(), value.float_val.end(), tmp.begin());
                 T2T(tmp.data(), data, len);
             } else {
                 std::vector<half> tmp(len);
                 for (size_t i = 0; i < len; ++i) {
-                    const uint16_t bits = value.half_val[i < listed ? i : listed - 1];
+                    const uint16_t bits = listed > 0 ? value.half_val[i < listed ? i : listed - 1] : (uint16_t) 0;
                     std::memcpy(&tmp[i], &bits, sizeof(bits));
                 }
                 T2T(tmp.data(), data, len);

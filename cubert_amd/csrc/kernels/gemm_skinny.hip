@@ -162,14 +162,16 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
 
 }  // namespace
 
-// Launches the kernel when the problem fits it, else returns CUBERT_UNSUPPORTED and launches nothing.
-// activation: 0 = none, 1 = erf-form GELU applied to alpha * A B + bias (the BertIntermediate layer).
-// `partials` holds partial_floats floats, `counters` n_counters ints that are zero between launches.
-// packed != 0: A is the output of gemm_skinny_pack for the same M and K (lda is ignored).
+// How a problem is cut: feature blocks, K slices and the chunks of 16 reduction values per slice.
+struct SkinnyPlan {
+    int blocks = 0, slices = 0, chunks_per_slice = 0;
+};
+
+// Every check gemm_skinny makes and the cut it would launch with; launches nothing.  Returns 0, CUBERT_BAD_ARGUMENT or
+// CUBERT_UNSUPPORTED exactly as gemm_skinny does for the same arguments.
 template <typename T>
-int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, int packed, const T *B, int ldb, T *C, int ldc,
-                const T *bias, int activation, float *partials, size_t partial_floats, int *counters,
-                int n_counters, hipStream_t stream) {
+int gemm_skinny_plan(int M, int N, int K, const T *A, int lda, int packed, const T *B, int ldb, int ldc, int activation,
+                     size_t partial_floats, int n_counters, SkinnyPlan *plan) {
     if (activation != 0 && activation != 1) return CUBERT_BAD_ARGUMENT;
     if (M <= 0 || N <= 0 || N > 32 || K <= 0 || K % kSkinnyChunk != 0) return CUBERT_UNSUPPORTED;
     if ((!packed && lda < M) || ldb < K || ldc < M) return CUBERT_BAD_ARGUMENT;
@@ -194,6 +196,22 @@ int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, int packe
         slices = (chunks + chunks_per_slice - 1) / chunks_per_slice;
     }
     if (blocks > 65535 || slices > 65535 || (slices > 1 && blocks > n_counters)) return CUBERT_UNSUPPORTED;
+    plan->blocks = blocks, plan->slices = slices, plan->chunks_per_slice = chunks_per_slice;
+    return 0;
+}
+
+// Launches the kernel when the problem fits it, else returns CUBERT_UNSUPPORTED and launches nothing.
+// activation: 0 = none, 1 = erf-form GELU applied to alpha * A B + bias (the BertIntermediate layer).
+// `partials` holds partial_floats floats, `counters` n_counters ints that are zero between launches.
+// packed != 0: A is the output of gemm_skinny_pack for the same M and K (lda is ignored).
+template <typename T>
+int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, int packed, const T *B, int ldb, T *C, int ldc,
+                const T *bias, int activation, float *partials, size_t partial_floats, int *counters,
+                int n_counters, hipStream_t stream) {
+    SkinnyPlan plan;
+    const int rc = gemm_skinny_plan<T>(M, N, K, A, lda, packed, B, ldb, ldc, activation, partial_floats, n_counters, &plan);
+    if (rc) return rc;
+    const int blocks = plan.blocks, slices = plan.slices, chunks_per_slice = plan.chunks_per_slice;
     const dim3 grid(blocks, slices), block(kSkinnyThreads);
 #define CUBERT_SKINNY_LAUNCH(GELU, PACKED)                                                                           \
     do {                                                                                                             \
@@ -292,13 +310,18 @@ int gemm_skinny_noalloc_f32(int M, int N, int K, float alpha, const float *A, in
     if (rc) return rc;
     float *partials = reinterpret_cast<float *>(base);
     int *counters = reinterpret_cast<int *>(base + kNoAllocPartialFloats * sizeof(float));
+    // Every argument and shape check first: a call that is refused has launched nothing (a caller that is capturing
+    // a graph records no stray node), exactly as cubert_gemm_skinny_f32.
+    SkinnyPlan plan;
+    const int refused = gemm_skinny_plan<float>(M, N, K, A, lda, 0, B, ldb, ldc, activation, kNoAllocPartialFloats,
+                                                kNoAllocCounters, &plan);
+    if (refused) return refused;
     // The array keeps what the last call left in it.  The partial tiles are written before they are read; the
     // counters must start at zero, so the ones this launch can touch are cleared first, on the same stream, by a
     // kernel (not a memset node, which a caller's graph capture would record).
-    const int blocks = M > 0 ? (M + 31) / 32 : 0;
-    if (blocks > 0 && blocks <= kNoAllocCounters) {
-        const int e = launch_untimed(zero_ints_kernel, dim3((blocks + kBlock - 1) / kBlock), dim3(kBlock), 0, stream,
-                                     counters, blocks);
+    if (plan.slices > 1) {
+        const int e = launch_untimed(zero_ints_kernel, dim3((plan.blocks + kBlock - 1) / kBlock), dim3(kBlock), 0, stream,
+                                     counters, plan.blocks);
         if (e) return e;
     }
     return gemm_skinny<float>(M, N, K, alpha, A, lda, 0, B, ldb, C, ldc, bias, activation, partials,

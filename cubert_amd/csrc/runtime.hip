@@ -388,13 +388,14 @@ int run_gemm(void *handle, int type, int transA, int transB, int M, int N, int K
     if (M == 0 || N == 0 || batch == 0) return 0;
     GemmKey key{type, transA, transB, M, N, K, lda, ldb, ldc, batch, strideA, strideB, strideC, bias != nullptr,
                 beta == 0.f};
+    // one launch at a time per context: the stream it launches on (cubert_blas_set_stream changes it under the same
+    // lock), the plan cache, and the few-token kernel's partial tiles and counters
+    std::lock_guard<std::mutex> lock(ctx->mutex);
     ctx->used = true;
     if (force_naive_gemm()) {
         return run_naive_gemm(ctx->stream, type, transA, transB, M, N, K, alpha, A, lda, strideA, B, ldb, strideB,
                               beta, C, ldc, strideC, batch, bias);
     }
-    // one launch at a time per context: the plan cache, and the few-token kernel's partial tiles and counters
-    std::lock_guard<std::mutex> lock(ctx->mutex);
     if (type != 2 && !transA && !transB && batch == 1 && beta == 0.f && N <= 32 && !library_gemm_only()) {
         const int rc = run_skinny(ctx, type, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, 0);
         if (rc != CUBERT_UNSUPPORTED) return rc;
@@ -459,6 +460,15 @@ void *cubert_malloc(size_t size) {
 }
 
 int cubert_free(void *ptr) { return ptr ? hip_rc(hipFree(ptr)) : 0; }
+
+int cubert_mem_info(size_t *free_bytes, size_t *total_bytes) {
+    size_t free_b = 0, total_b = 0;
+    const hipError_t e = hipMemGetInfo(&free_b, &total_b);
+    if (e != hipSuccess) return (int) e;
+    if (free_bytes != nullptr) *free_bytes = free_b;
+    if (total_bytes != nullptr) *total_bytes = total_b;
+    return 0;
+}
 
 int cubert_memcpy(void *dst, const void *src, size_t n, int kind) {
     if (n == 0) return 0;
@@ -608,6 +618,8 @@ int cubert_gemm_skinny_f16(void *handle, int M, int N, int K, float alpha, const
 
 int cubert_gemm_skinny_noalloc_f32(void *stream, int M, int N, int K, float alpha, const float *A, int lda,
                                    const float *B, int ldb, float *C, int ldc, const float *bias, int activation) {
+    if (!A || !B || !C) return CUBERT_BAD_ARGUMENT;
+    if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;  // as cubert_gemm_skinny_f32
     return cubert::gemm_skinny_noalloc_f32(M, N, K, alpha, A, lda, B, ldb, C, ldc, bias, activation,
                                            (hipStream_t) stream);
 }

@@ -63,7 +63,10 @@ int cubert_model_info(void *model, int compute_type, int *hidden_size, int *num_
  * src/cuBERT/tensorflow/Graph.h:10-23, Graph.cpp:13-91: the float and binary16 constants of a frozen GraphDef
  * converted to dtype (0 float, 1 binary16), by node name.  CPU only.  cubert_graph_var gives the host pointer the
  * graph owns (NULL for an unknown name), the number of elements it holds and, when dims != NULL, up to max_dims
- * dimensions of the declared shape (*n_dims receives the rank).  cubert_graph_sizes gives vocab_size,
+ * dimensions of the declared shape (*n_dims receives the rank).  The dimensions are the file's declaration, the
+ * element count is what the file holds (bytes of tensor_content; a value list repeated up to the declared size; a
+ * declared shape with no data at all read as zeros): the two may disagree for a malformed file, as in the reference
+ * (Graph.cpp:50-56), and a model is checked against the shapes it needs when it is built.  cubert_graph_sizes gives vocab_size,
  * type_vocab_size, hidden_size, intermediate_size and num_labels in that order. */
 int cubert_graph_open(const char *model_file, int dtype, void **graph);
 long long cubert_graph_count(void *graph, int dtype);

@@ -192,6 +192,10 @@ int cubert_gpu_info(int device); /* prints name, memory and clock to stderr */
 
 void *cubert_malloc(size_t size); /* device memory; NULL on failure */
 int cubert_free(void *ptr);
+/* Free and total device memory of the current GPU in bytes (either pointer may be NULL): what the reference prints
+ * when an allocation fails (src/cuBERT/common.cpp:158-161), here also readable by a caller that wants to see what a
+ * model or a call took. */
+int cubert_mem_info(size_t *free_bytes, size_t *total_bytes);
 /* kind: 1 host->device, 2 device->host, 3 device->device (cudaMemcpyKind numbering, common.h:31-40) */
 int cubert_memcpy(void *dst, const void *src, size_t n, int kind);
 int cubert_memcpy_async(void *dst, const void *src, size_t n, int kind, void *stream);

@@ -11,7 +11,8 @@ serialise a GraphDef the way TensorFlow's freeze_graph writes one:
     one of them stored as DT_HALF;
   * scalar constants in float_val and half_val, packed (proto3 default) and unpacked (second message set whose
     repeated scalars are declared [packed = false]; the wire format allows both and parsers must accept both);
-  * a splat (shape [5], one float_val), a one-element vector in float_val, an empty Const;
+  * a splat (shape [5], one float_val), a one-element vector in float_val, an empty Const, all-zero tensors
+    written as a bare shape (what TensorFlow's tensor compression leaves of them);
   * nodes that are not weights: Placeholder, MatMul with bool/type attrs, an op with a float attr (fixed32),
     int32 Consts in tensor_content and int_val, a node whose attr "value" is a string, a list attr;
   * GraphDef.versions, GraphDef.version and a GraphDef.library whose FunctionDef holds a Const named like a
@@ -234,6 +235,11 @@ def build():
     expected["loss/one_element_bias"] = np.array([0.125], np.float32)
     _const(g, "bert/encoder/empty", DT_FLOAT, [0])
     expected["bert/encoder/empty"] = np.zeros(0, np.float32)
+    # an all-zero tensor after TensorFlow's tensor compression: a shape, no tensor_content and no value list
+    _const(g, "bert/encoder/zeros_compressed", DT_FLOAT, [2, 3])
+    expected["bert/encoder/zeros_compressed"] = np.zeros(6, np.float32)
+    _const(g, "bert/encoder/zeros_compressed_half", DT_HALF, [4])
+    expected["bert/encoder/zeros_compressed_half"] = np.zeros(4, np.float32)
 
     # a repeated name: the later node wins
     _const(g, "repeated/name", DT_FLOAT, [2], content=np.array([1, 2], np.float32).tobytes())

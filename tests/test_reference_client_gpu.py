@@ -118,3 +118,89 @@ def test_reference_python_extension_links_against_this_library():
     r = subprocess.run(["ldd", "-r", PY_EXTENSION[0]], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     unresolved = [l for l in r.stdout.splitlines() if "undefined symbol" in l and "Py" not in l and "_Py" not in l]
     assert not unresolved, unresolved
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("compute_type", [0, 1])
+def test_public_symbols_driven_the_way_the_reference_python_binding_drives_them(tmp_path, compute_type):
+    """The calls python/cuBERT.pyx makes, in its order, on the exported cuBERT_* symbols themselves (not the
+    exception-free cubert_try_* forms the package uses): cuBERT_initialize at import (cuBERT.pyx:9),
+    cuBERT_open then cuBERT_open_tokenizer (:121-138), cuBERT_compute_m and cuBERT_tokenize_compute_m with a
+    cuBERT_Output whose five pointers sit in the header's order and of which only some are set (:41-114,171-177,
+    202-208), cuBERT_close then cuBERT_close_tokenizer (:140-143), cuBERT_finalize (:10).  Outputs carry the
+    model's element type (half for a half model).  The argument-error paths are C++ exceptions there (`except +`
+    in _cuBERT.pxd) and cannot cross ctypes; they are covered through cubert_try_* in the model tests."""
+    import ctypes
+    from cubert_amd._lib import LIB_PATH, cuBERT_Output
+    from cubert_amd.graphdef import write_graphdef
+    from cubert_amd.testing import random_bert_weights, random_inputs
+    from oracle import tokenizer as otok
+    cfg = dict(vocab=211, hidden=128, layers=3, heads=4, intermediate=512, max_position=64, type_vocab=2)
+    w = random_bert_weights(seed=5, labels=2, ln_random=True, **cfg)
+    write_graphdef(str(tmp_path / "model.pb"), w)
+    lines = ["[PAD]", "[UNK]", "[CLS]", "[SEP]"] + list("abcdefghijklmnopqrstuvwxyz") + ["##" + c for c in "abcdefgh"]
+    (tmp_path / "vocab.txt").write_text("\n".join(lines) + "\n", encoding="utf8")
+
+    L = ctypes.CDLL(LIB_PATH)  # a second handle on the same library, with the signatures of _cuBERT.pxd only
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    L.cuBERT_open.restype, L.cuBERT_open.argtypes = vp, [ctypes.c_char_p, ci, ci, ci, ci, ci]
+    L.cuBERT_open_tokenizer.restype, L.cuBERT_open_tokenizer.argtypes = vp, [ctypes.c_char_p, ci]
+    L.cuBERT_compute_m.restype = None
+    L.cuBERT_compute_m.argtypes = [vp, ci, vp, vp, vp, ctypes.POINTER(cuBERT_Output), ci, ci]
+    L.cuBERT_tokenize_compute_m.restype = None
+    L.cuBERT_tokenize_compute_m.argtypes = [vp, vp, ci, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(ctypes.c_char_p),
+                                            ctypes.POINTER(cuBERT_Output), ci, ci]
+    L.cuBERT_close.restype, L.cuBERT_close.argtypes = None, [vp, ci]
+    L.cuBERT_close_tokenizer.restype, L.cuBERT_close_tokenizer.argtypes = None, [vp]
+    L.cuBERT_get_gpu_count.restype = ci
+
+    assert [name for name, _ in cuBERT_Output._fields_] == ["logits", "pooled_output", "sequence_output",
+                                                            "embedding_output", "probs"]
+    assert ctypes.sizeof(cuBERT_Output) == 5 * ctypes.sizeof(vp)
+
+    half = compute_type == 1
+    dt = np.float16 if half else np.float32
+    tol = 1e-2 if half else 1e-5
+    wf = {k: oracle.round_to_half(v) for k, v in w.items()} if half else w
+
+    L.cuBERT_initialize()
+    assert L.cuBERT_get_gpu_count() >= 1
+    model = L.cuBERT_open(str(tmp_path / "model.pb").encode(), 4, 32, cfg["layers"], cfg["heads"], compute_type)
+    tokenizer = L.cuBERT_open_tokenizer(str(tmp_path / "vocab.txt").encode(), 1)
+    assert model and tokenizer
+
+    ids, mask, seg = random_inputs(seed=6, batch=3, seq_length=32, vocab=cfg["vocab"], min_valid=4, segment_split=9)
+    want = oracle.bert_forward(wf, ids, mask, seg, cfg["layers"], cfg["heads"])
+    pooled, probs = np.full((3, 128), np.nan, dt), np.full((3, 2), np.nan, dt)
+    out = cuBERT_Output(None, pooled.ctypes.data, None, None, probs.ctypes.data)   # Output(pooled_output=..., probs=...)
+    L.cuBERT_compute_m(model, 3, ids.ctypes.data, mask.ctypes.data, seg.ctypes.data, ctypes.byref(out), compute_type, 0)
+    assert_close(pooled.astype(np.float32), want["pooled_output"], tol, "pooled_output")
+    assert_close(probs.astype(np.float32), want["probs"], tol, "probs")
+
+    # Output(sequence_output) alone, the way compute() wraps one array (cuBERT.pyx:147-156)
+    sequence = np.full((3, 32, 128), np.nan, dt)
+    out = cuBERT_Output(None, None, sequence.ctypes.data, None, None)
+    L.cuBERT_compute_m(model, 3, ids.ctypes.data, mask.ctypes.data, seg.ctypes.data, ctypes.byref(out), compute_type, 0)
+    if half:   # token-level bound of the model tests: 1e-2 * max(1, |x|)
+        assert np.all(np.abs(sequence.astype(np.float32) - want["sequence_output"]) <=
+                      1e-2 * np.maximum(1.0, np.abs(want["sequence_output"])))
+    else:
+        assert_close(sequence, want["sequence_output"], tol, "sequence_output")
+
+    text_a, text_b = ["abc def", "hello again", "x"], ["gh", "", "zzz yx"]
+    vocab = otok.load_vocab(lines)
+    feats = [otok.convert_single_example(vocab, 32, a, b) for a, b in zip(text_a, text_b)]
+    t_ids = np.array([f[0] for f in feats], np.int32)
+    t_mask = np.array([f[1] for f in feats], np.int8)
+    t_seg = np.array([f[2] for f in feats], np.int8)
+    want = oracle.bert_forward(wf, t_ids, t_mask, t_seg, cfg["layers"], cfg["heads"])
+    arr_a = (ctypes.c_char_p * 3)(*[s.encode() for s in text_a])
+    arr_b = (ctypes.c_char_p * 3)(*[s.encode() for s in text_b])
+    logits = np.full((3, 2), np.nan, dt)
+    out = cuBERT_Output(logits.ctypes.data, None, None, None, None)
+    L.cuBERT_tokenize_compute_m(model, tokenizer, 3, arr_a, arr_b, ctypes.byref(out), compute_type, 0)
+    assert_close(logits.astype(np.float32), want["logits"], tol, "logits from texts")
+
+    L.cuBERT_close(model, compute_type)
+    L.cuBERT_close_tokenizer(tokenizer)
+    L.cuBERT_finalize()

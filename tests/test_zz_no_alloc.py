@@ -100,6 +100,38 @@ def test_two_calls_in_a_row_the_second_smaller(L, context):
     run_pair(L, handle, stream, 40, 1, 16, 0, seed=5)          # one slice: no scratch at all, ragged feature block
 
 
+def free_device_bytes(L):
+    free = ctypes.c_size_t()
+    assert L.cubert_mem_info(ctypes.byref(free), None) == 0
+    return free.value
+
+
+def test_calls_leave_free_device_memory_unchanged(L, context):
+    """The headline property: after the first call on the device (which looks up the array's address) no call
+    changes the amount of free device memory, whether it launches, is refused for its shape or for its size."""
+    _, stream = context
+    rng = np.random.default_rng(11)
+    M, N, K = 768, 32, 3072
+    A = rng.normal(0, 0.05, (K, M)).astype(np.float32)
+    B = rng.normal(0, 1.0, (N, K)).astype(np.float32)
+    d = Device(L, A, B, np.zeros((N, M), np.float32))
+
+    def call(m, n, k):
+        return L.cubert_gemm_skinny_noalloc_f32(stream, m, n, k, 1.0, d.ptrs[0], m, d.ptrs[1], k, d.ptrs[2], m, None, 0)
+
+    assert call(M, N, K) == 0                       # first call: set-up done
+    assert L.cubert_stream_synchronize(stream) == 0
+    before = free_device_bytes(L)
+    for _ in range(20):
+        assert call(M, N, K) == 0
+        assert call(96, 5, 256) == 0
+        assert call(32, 33, 16) == UNSUPPORTED
+    assert call(NOALLOC_MAX_M + 1, 1, 16) == TOO_LARGE
+    assert L.cubert_stream_synchronize(stream) == 0
+    assert free_device_bytes(L) == before
+    d.free()
+
+
 def test_back_to_back_launches_without_a_wait_between(L, context):
     """Ten launches of alternating shapes queued on one stream before anything is waited for: each finds the counters
     cleared and its partial tiles its own."""
