@@ -44,6 +44,8 @@ SIGNATURES = {
     "cubert_try_close": (ci, [vp, ci]),
     "cubert_model_info": (ci, [vp, ci, ctypes.POINTER(ci), ctypes.POINTER(ci), ctypes.POINTER(ci)]),
     "cubert_check_input_range": (ci, [vp, vp, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t]),
+    "cubert_open_warmup_batches": (cll, [ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t),
+                                         ctypes.c_size_t]),
     "cubert_graph_open": (ci, [ctypes.c_char_p, ci, ctypes.POINTER(vp)]),
     "cubert_graph_count": (cll, [vp, ci]),
     "cubert_graph_var": (vp, [vp, ci, ctypes.c_char_p, ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(cll), ci,

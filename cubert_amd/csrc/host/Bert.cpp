@@ -40,6 +40,52 @@ void check_input_range(const int *input_ids, const int8_t *segment_ids, size_t c
     }
 }
 
+// Batch sizes to prepare when a model is opened, from CUBERT_OPEN_WARMUP: unset = the maximum batch only (what the
+// reference prepares, src/cuBERT/Bert.cpp:62-64); "0" = none; otherwise a comma-separated list of batch sizes, in
+// which "max" stands for max_batch_size ("1,8,max").  Entries that are not a size in [1, max_batch_size] are named
+// on stderr and skipped.
+std::vector<size_t> open_warmup_batches(const char *setting, size_t max_batch_size) {
+    std::vector<size_t> batches;
+    if (setting == nullptr) {
+        batches.push_back(max_batch_size);
+        return batches;
+    }
+    const std::string text(setting);
+    if (text == "0") return batches;
+    size_t at = 0;
+    while (at <= text.size()) {
+        size_t end = text.find(',', at);
+        if (end == std::string::npos) end = text.size();
+        std::string item = text.substr(at, end - at);
+        at = end + 1;
+        while (!item.empty() && (item.back() == ' ' || item.back() == '\t')) item.pop_back();
+        while (!item.empty() && (item.front() == ' ' || item.front() == '\t')) item.erase(item.begin());
+        if (item.empty()) continue;
+        size_t batch = 0;
+        bool ok = true;
+        if (item == "max") {
+            batch = max_batch_size;
+        } else {
+            for (char c : item) {
+                if (c < '0' || c > '9' || batch > (size_t) 1 << 40) {
+                    ok = false;
+                    break;
+                }
+                batch = batch * 10 + (size_t) (c - '0');
+            }
+        }
+        if (!ok || batch == 0 || batch > max_batch_size) {
+            std::cerr << "cuBERT: CUBERT_OPEN_WARMUP entry \"" << item << "\" is not a batch size in [1, " << max_batch_size
+                      << "]; skipped" << std::endl;
+            continue;
+        }
+        bool seen = false;
+        for (size_t b : batches) seen = seen || b == batch;
+        if (!seen) batches.push_back(batch);
+    }
+    return batches;
+}
+
 template <typename T>
 Bert<T>::Bert(const std::unordered_map<std::string, T *> &var, size_t max_batch_size, size_t seq_length,
               size_t vocab_size, size_t type_vocab_size, size_t hidden_size, size_t num_hidden_layers,
@@ -89,8 +135,7 @@ Bert<T>::Bert(const std::unordered_map<std::string, T *> &var, size_t max_batch_
         output_staging = static_cast<unsigned char *>(cubert_malloc_host(kOutputStagingBytes));
         if (output_staging == nullptr) throw std::runtime_error("no page-locked host memory for the outputs");
 
-        const char *warm = std::getenv("CUBERT_OPEN_WARMUP");
-        if (warm == nullptr || std::string(warm) != "0") _pre_compute(max_batch_size);
+        for (size_t batch : open_warmup_batches(std::getenv("CUBERT_OPEN_WARMUP"), max_batch_size)) _pre_compute(batch);
     } catch (...) {
         release();
         throw;

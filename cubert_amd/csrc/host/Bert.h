@@ -22,6 +22,10 @@ namespace cuBERT {
 void check_input_range(const int *input_ids, const int8_t *segment_ids, size_t count, size_t vocab_size,
                        size_t type_vocab_size);
 
+// The batch sizes a model prepares when it is opened, read from the text of CUBERT_OPEN_WARMUP (nullptr = unset):
+// unset = max_batch_size only, "0" = none, else a comma-separated list in which "max" stands for max_batch_size.
+std::vector<size_t> open_warmup_batches(const char *setting, size_t max_batch_size);
+
 template <typename T>
 class Bert {
 public:
@@ -39,7 +43,8 @@ public:
 
     // One forward pass of `batch_size` sequences on made-up inputs: plans (and where it applies times) every GEMM
     // shape of that batch size, so that the first request of that size does not pay for it.  The constructor runs
-    // it for max_batch_size (CUBERT_OPEN_WARMUP=0 in the environment skips that).  Nothing needs preparing
+    // it for max_batch_size (CUBERT_OPEN_WARMUP=0 in the environment skips that, a list such as 1,8,max names the
+    // batch sizes to prepare instead).  Nothing needs preparing
     // between requests, unlike in the reference, whose _pre_compute refills the Dense outputs with their biases.
     void _pre_compute(size_t batch_size);
 

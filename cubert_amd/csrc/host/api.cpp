@@ -425,6 +425,12 @@ int cubert_check_input_range(const int *input_ids, const int8_t *segment_ids, si
     });
 }
 
+long long cubert_open_warmup_batches(const char *setting, size_t max_batch_size, size_t *batches, size_t capacity) {
+    const std::vector<size_t> found = cuBERT::open_warmup_batches(setting, max_batch_size);
+    for (size_t i = 0; i < found.size() && i < capacity && batches != nullptr; ++i) batches[i] = found[i];
+    return (long long) found.size();
+}
+
 int cubert_graph_open(const char *model_file, int dtype, void **graph) {
     return guarded([&] {
         if (graph == nullptr || model_file == nullptr) throw std::invalid_argument("null argument");

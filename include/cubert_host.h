@@ -55,6 +55,13 @@ int cubert_try_compute_m(void *model, int batch_size, int *input_ids, int8_t *in
  * first offender otherwise.  (The reference indexes its tables unchecked, src/cuBERT/op/Embedding.cpp:16-19.) */
 int cubert_check_input_range(const int *input_ids, const int8_t *segment_ids, size_t count, size_t vocab_size,
                              size_t type_vocab_size);
+/* The batch sizes a model prepares when it is opened (one forward pass each on made-up inputs, so that a first
+ * request of that size does not pay for GEMM planning), as read from the text of the environment variable
+ * CUBERT_OPEN_WARMUP (`setting`, NULL = unset): unset = max_batch_size only, which is what the reference prepares
+ * (src/cuBERT/Bert.cpp:62-64); "0" = none; else a comma-separated list of batch sizes in which "max" stands for
+ * max_batch_size, e.g. "1,8,max".  Entries outside [1, max_batch_size] are named on stderr and skipped.  Writes up
+ * to `capacity` sizes to `batches` in the order they will run and returns how many there are.  CPU only. */
+long long cubert_open_warmup_batches(const char *setting, size_t max_batch_size, size_t *batches, size_t capacity);
 /* replaces: cuBERT_close, reference src/cuBERT.cpp:92-102 */
 int cubert_try_close(void *model, int compute_type);
 /* Shape facts of an opened model (hidden size, labels, seq_length) for sizing output arrays. */

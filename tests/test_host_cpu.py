@@ -257,6 +257,29 @@ def test_input_range_check():
     assert check(big, np.zeros(big.size, np.int8), (1 << 15) - 1, 2)[0] == 1
 
 
+def test_open_warmup_batch_list():
+    """CUBERT_OPEN_WARMUP as a model reads it when it is opened: unset = the maximum batch (what the reference
+    prepares, src/cuBERT/Bert.cpp:62-64), "0" = nothing, else a list of batch sizes with "max" for the maximum."""
+    import ctypes
+    from cubert_amd._lib import lib
+    L = lib()
+
+    def batches(setting, max_batch):
+        out = (ctypes.c_size_t * 16)()
+        n = L.cubert_open_warmup_batches(None if setting is None else setting.encode(), max_batch, out, 16)
+        return [out[i] for i in range(min(n, 16))]
+
+    assert batches(None, 128) == [128]
+    assert batches("0", 128) == []
+    assert batches("", 128) == []
+    assert batches("1,8,32", 128) == [1, 8, 32]
+    assert batches(" 8 , max,1,8", 128) == [8, 128, 1]          # order kept, repeats dropped
+    assert batches("1", 128) == [1]
+    assert batches("max", 4) == [4]
+    assert batches("1,129,0,x,-3,16", 128) == [1, 16]           # the others are named on stderr and skipped
+    assert batches("99999999999999999999999", 128) == []
+
+
 def test_bench_refuses_more_than_one_gpu():
     """This build measures one GPU: `bench.py --gpus N` with N > 1 exits with a message instead of a number."""
     import subprocess

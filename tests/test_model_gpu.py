@@ -510,6 +510,32 @@ def test_first_request_does_not_pay_for_gemm_planning(cb):
     assert_close(out.pooled_output[:4], want, FP32_TOL, "pooled output after the timed requests")
 
 
+def test_listed_batch_sizes_are_prepared_at_open(cb, monkeypatch):
+    """CUBERT_OPEN_WARMUP=48,max: the model prepares batch 48 as well as its maximum when it is opened, so the first
+    request of 48 sequences (1536 tokens: library GEMMs of 1.8 ... 7 GFLOP, chosen by timing) costs what later ones
+    cost; results are those of the oracle."""
+    import time
+    from cubert_amd.testing import BERT_BASE, random_bert_weights, random_inputs
+    shape = dict(BERT_BASE, layers=2, vocab=1000, max_position=32)
+    w = random_bert_weights(seed=15, labels=2, **shape)
+    ids, mask, seg = random_inputs(seed=16, batch=48, seq_length=32, vocab=1000, min_valid=8)
+    monkeypatch.setenv("CUBERT_OPEN_WARMUP", "48,max")
+    bert = cb.Bert(w, 96, 32, 2, 12)
+    out = cb.Output(np.empty((48, 768), np.float32), cb.OutputType.POOLED_OUTPUT)
+    times = []
+    for _ in range(6):
+        t = time.perf_counter()
+        bert.compute(ids, mask, seg)
+        bert.output(48, out)
+        times.append((time.perf_counter() - t) * 1e3)
+    bert.close()
+    later = float(np.median(times[1:]))
+    print("\nfirst request of a listed size %.2f ms, later requests %.2f ms (median of 5)" % (times[0], later))
+    assert times[0] <= 3 * later + 2.0, times
+    want = oracle.bert_forward(w, ids[:4], mask[:4], seg[:4], 2, 12)["pooled_output"]
+    assert_close(out.pooled_output[:4], want, FP32_TOL, "pooled output after the timed requests")
+
+
 def test_api_error_behaviour(cb, small_pb):
     path, _ = small_pb
     with pytest.raises(ValueError, match="model file not found"):
