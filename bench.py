@@ -6,13 +6,19 @@
 A step is one forward pass of the workload (default C1: BERT-base fp32, batch 128, seq_len 32,
 the configuration the headline metric is quoted on) on inputs already resident in device memory.
 Prints ONE JSON line:
-  value / ms_per_step   sequences/s over the K timed device-resident steps
-  roofline              the dominant fused kernel (bias+GELU), HIP events around its launches inside the timed steps
+  value / ms_per_step   sequences/s over the K timed device-resident steps (inputs already in HBM when the timed
+                        region starts)
+  reference_protocol    the same workload the way the reference's benchmark client measures it
+                        (benchmark/benchmark_cu.cpp:68-78): host arrays in, POOLED_OUTPUT host array out, 10 warm-up
+                        calls, then max(K, 50) timed calls, PCIe-inclusive; mean and p50 per call, sequences/s
+  p50_ms_batch1_host_path   the same call with one sequence: the latency half of the headline metric
+  roofline              the dominant fused kernel (bias+GELU), HIP events carried by its launches inside the timed steps
   kernels               every kernel kind of the forward pass: average launch time, GB/s, fraction of the HBM peak
-  clean_roofline        the same table at C3 (BERT-base fp16, batch 64, seq_len 512), whose tensors do not fit the
+                        (the dominant kernel's row is the `roofline` measurement: one timing per kernel)
+  gemm                  the Dense GEMMs one by one and in total: FLOPs, average microseconds, TFLOP/s and the fraction
+                        of the matrix-core peak of the arithmetic type (fp32 157.3 TFLOP/s, fp16 2.5 PFLOP/s)
+  clean_roofline        `kernels` and `gemm` at C3 (BERT-base fp16, batch 64, seq_len 512), whose tensors do not fit the
                         256 MB Infinity Cache: the workload where a fraction of the HBM peak is an HBM statement
-  host_path             the reference benchmark client's protocol (benchmark/benchmark_cu.cpp:68-78): host arrays in,
-                        POOLED_OUTPUT out, 10 warm-up calls, then timed calls (PCIe-inclusive)
   cpu_baseline          the CPU oracle on this host's cores on a bounded sample of the same workload, with the
                         thread counts the libraries report and the time per part of a pass
 """
@@ -30,6 +36,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"f32": 157.3, "f16": 2500.0}  # dense matrix-core peaks of the part, by operand type
+# How a launch's event pair reads against a profiler's kernel duration (measured on bias+GELU at C1: 17.2-17.4 us by
+# the pair, 15.9-16.4 us by rocprofv3 in profiles/forward_C1_kernel_stats.md): fractions computed from event pairs are
+# the lower of the two.
+EVENT_PAIR_NOTE = ("HIP event pair carried by each launch (start/stop of the dispatch); reads 1-1.5 us above "
+                   "rocprofv3's kernel duration for the same launch, so fractions from it are the conservative ones")
 
 # Bytes per launch that crossed the L2 <-> memory boundary, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script scaled by a plain copy of known size (method and table: profiles/traffic_pmc.md).  Hardware counters
@@ -203,11 +215,68 @@ def standalone_kernel(kind, cfg, mask, alg_bytes, reps=20):
                     "another kernel (%s)" % ("attention_fused" if kind == "mask_scale_softmax" else "the few-token Dense")}
 
 
+def dense_flops(cfg):
+    """{Dense kind: (FLOPs per launch, launches per forward pass, out features, tokens, in features)}."""
+    m = cfg["model"]
+    B, S = cfg["batch"], cfg["seq_length"]
+    H, I, L = m["hidden"], m["intermediate"], m["layers"]
+    M = B * S
+    shapes = {"dense_qkv": (3 * H, M, H, L), "dense_attention_output": (H, M, H, L),
+              "dense_intermediate": (I, M, H, L), "dense_output": (H, M, I, L), "dense_pooler": (H, B, H, 1)}
+    return {k: (2.0 * n * t * kk, count, n, t, kk) for k, (n, t, kk, count) in shapes.items()}
+
+
+def gemm_table(bert, cfg, batch, passes, ms_per_step, kernels, kernel_passes):
+    """The Dense GEMMs one by one, from `passes` extra forward passes in which only they are timed: FLOPs, average
+    microseconds, TFLOP/s, fraction of the matrix-core peak of the operand type, and the total per forward pass.
+    A library call may be several launches, so it sits between two marker events, and that interval also holds the
+    gaps to the neighbouring kernels: these times are upper bounds (their sum over a pass plus the other kernels
+    exceeds the step time).  `total.by_difference` is the lower bound: the step time minus the event-pair times of
+    every other kernel of a pass (`kernels`, measured over `kernel_passes` passes).  The exact durations are the
+    profiler's, profiles/forward_*_kernel_stats.md."""
+    peak = MFMA_PEAK_TFLOPS[cfg["dtype"]]
+    e = 4 if cfg["dtype"] == "f32" else 2
+    flops = dense_flops(cfg)
+    bert.profile(list(bert.DENSE_KINDS))
+    for _ in range(passes):
+        bert.compute_resident(batch)
+    read = bert.profile_read()
+    bert.profile([])
+    rows, total_flop, total_ms = {}, 0.0, 0.0
+    for k in bert.DENSE_KINDS:
+        if k not in read:
+            continue
+        ms, n = read[k]
+        us = ms * 1e3 / n
+        fl, per_pass, out_f, tokens, in_f = flops[k]
+        tf = fl / (us * 1e-6) / 1e12
+        rows[k] = {"out_features": out_f, "tokens": tokens, "in_features": in_f, "GFLOP": round(fl / 1e9, 3),
+                   "avg_us": round(us, 2), "launches": n, "TFLOP/s": round(tf, 2), "frac_mfma_peak": round(tf / peak, 4),
+                   "weights_GB/s": round(out_f * in_f * e / (us * 1e-6) / 1e9, 1)}
+        total_flop += fl * per_pass
+        total_ms += ms / passes
+    tf = total_flop / (total_ms * 1e-3) / 1e12 if total_ms > 0 else 0.0
+    others_ms = sum(row["avg_us"] * 1e-3 * row["launches"] / kernel_passes for k, row in kernels.items()
+                    if "note" not in row and k != "dense_gemm")
+    rest_ms = ms_per_step - others_ms
+    tf_rest = total_flop / (rest_ms * 1e-3) / 1e12 if rest_ms > 0 else 0.0
+    return {"peak_TFLOP/s": peak, "operands": cfg["dtype"], "accumulate": "f32", "shapes": rows,
+            "total": {"GFLOP_per_pass": round(total_flop / 1e9, 2), "ms_per_pass": round(total_ms, 4),
+                      "TFLOP/s": round(tf, 2), "frac_mfma_peak": round(tf / peak, 4),
+                      "by_difference": {"ms_per_pass": round(rest_ms, 4), "TFLOP/s": round(tf_rest, 2),
+                                        "frac_mfma_peak": round(tf_rest / peak, 4),
+                                        "share_of_step": round(rest_ms / ms_per_step, 4) if ms_per_step else None}},
+            "timing": "per shape and `total`: marker events around each library call inside full forward passes "
+                      "(includes the gaps to the neighbouring kernels: time is an upper bound, TFLOP/s a lower bound); "
+                      "`by_difference`: step time minus the event-pair times of all other kernels of a pass (time is a "
+                      "lower bound, TFLOP/s an upper bound)"}
+
+
 def kernel_table(bert, cfg, mask, alg, batch, passes):
     """Every kernel kind of `passes` forward passes with an event pair around each launch:
     {kind: average microseconds, launches, and for the fused kernels GB/s and fraction of the HBM peak}."""
     table = {}
-    bert.profile([k for k in bert.KINDS])
+    bert.profile([k for k in bert.KINDS if k not in bert.DENSE_KINDS])
     for _ in range(passes):
         bert.compute_resident(batch)
     for k, (ms, n) in bert.profile_read().items():
@@ -382,10 +451,17 @@ def main():
     achieved = alg[dominant] / (avg_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
-                "algorithmic_bytes_per_launch": alg[dominant], "avg_launch_us": round(avg_us, 2), "launches": launches}
+                "algorithmic_bytes_per_launch": alg[dominant], "avg_launch_us": round(avg_us, 2), "launches": launches,
+                "timing": EVENT_PAIR_NOTE + "; launches inside the timed steps"}
 
     # ---- every kernel kind, in extra untimed passes (reported, not part of `value`)
-    kernels = kernel_table(bert, cfg, mask, alg, B, max(5, args.steps // 5))
+    table_passes = max(5, args.steps // 5)
+    kernels = kernel_table(bert, cfg, mask, alg, B, table_passes)
+    gemm = gemm_table(bert, cfg, B, table_passes, ms_per_step, kernels, table_passes)
+    if dominant in prof:
+        # one timing per kernel: the dominant kernel's row is the measurement `roofline` reports
+        kernels[dominant] = {"avg_us": roofline["avg_launch_us"], "launches": launches, "GB/s": roofline["achieved"],
+                             "frac_hbm_peak": roofline["frac"], "source": "the timed steps (same figures as `roofline`)"}
 
     # ---- the public path: host arrays in, host array out (PCIe-inclusive), and p50 latency at batch 1
     host_path, p50_b1 = None, None
@@ -393,13 +469,17 @@ def main():
         out = np.empty((B, m["hidden"]), np.float16 if half else np.float32)
         o = cubert_amd.Output(out, cubert_amd.OutputType.POOLED_OUTPUT)
         lat = []
-        for i in range(10 + 50):  # 10 warm-up calls as the reference's benchmark client, then 50 timed
+        calls = max(args.steps, 50)
+        for i in range(10 + calls):  # 10 warm-up calls as the reference's benchmark client, then the timed ones
             t = time.perf_counter()
             bert.compute(ids, mask, seg)
             bert.output(B, o)
             if i >= 10:
                 lat.append((time.perf_counter() - t) * 1e3)
-        host_path = {"mean_ms": round(float(np.mean(lat)), 3), "p50_ms": round(float(np.median(lat)), 3),
+        host_path = {"protocol": "benchmark/benchmark_cu.cpp:68-78 of the reference: host arrays in, POOLED_OUTPUT host "
+                                 "array out per call (PCIe-inclusive), 10 warm-up calls, then the timed calls",
+                     "warmup_calls": 10, "timed_calls": calls,
+                     "mean_ms": round(float(np.mean(lat)), 3), "p50_ms": round(float(np.median(lat)), 3),
                      "sequences_per_s": round(B / (np.mean(lat) * 1e-3), 1), "output": "POOLED_OUTPUT"}
         lat1 = []
         for i in range(20 + 100):
@@ -429,13 +509,14 @@ def main():
         ms3 = (time.perf_counter() - t0) * 1e3 / 10
         alg3 = algorithmic_bytes(c3)
         table3 = kernel_table(big, c3, mask3, alg3, c3["batch"], 5)
+        gemm3 = gemm_table(big, c3, c3["batch"], 5, ms3, table3, 5)
         big.close()
         for k, row in table3.items():
             row["traffic"], _ = recorded_traffic("C3", k)
         clean = {"workload": "C3: BERT-base f16 batch %d seq_len %d, valid length min(512, 16 + Exp(96)), inputs "
                              "resident in HBM" % (c3["batch"], c3["seq_length"]),
                  "ms_per_step": round(ms3, 4), "sequences_per_s": round(c3["batch"] / (ms3 * 1e-3), 1), "steps": 10,
-                 "kernels": table3}
+                 "kernels": table3, "gemm": gemm3, "kernel_timing": EVENT_PAIR_NOTE}
 
     # ---- the same steps with the opt-in two-term fp16 Dense form of fp32 models (reported beside `value`, never as it)
     two_term = None
@@ -506,10 +587,12 @@ def main():
         "dtype": cfg["dtype"], "data": "synthetic",
         "config": {"workload": "%s: %s %s batch %d seq_len %d, random-init N(0,0.02) weights, inputs resident in HBM" %
                                (args.workload, "BERT-large" if m["hidden"] == 1024 else "BERT-base", cfg["dtype"], B, S),
-                   "value_is": "device-resident forward passes; the host-arrays-in / host-array-out protocol of the "
-                               "reference's benchmark client is `host_path`"},
+                   "value_is": "forward passes on inputs already resident in HBM (what this bench's contract defines "
+                               "`value` as; a PCIe-inclusive rate is never `value`). The same workload measured the way "
+                               "the reference's benchmark client does it (host arrays in, host array out) is "
+                               "`reference_protocol`, and `p50_ms_batch1_host_path` is that call with one sequence."},
+        "reference_protocol": host_path, "p50_ms_batch1_host_path": p50_b1,
         "roofline": roofline, "cpu_baseline": cpu,
-        "p50_ms_batch1_host_path": p50_b1, "host_path": host_path,
     }
     if two_term_dense() and not half:
         line["dtype"] = "f32 storage and accumulation; Dense products as three f16 matrix-core products of two-term operands"
@@ -520,6 +603,8 @@ def main():
     for k, row in kernels.items():
         row["traffic"], _ = recorded_traffic(args.workload, k)
     line["kernels"] = kernels
+    line["kernel_timing"] = EVENT_PAIR_NOTE
+    line["gemm"] = gemm
     if clean is not None:
         line["clean_roofline"] = clean
     print(json.dumps(line))

@@ -349,7 +349,10 @@ class Bert(object):
             raise RuntimeError("stream synchronize failed: %d" % rc)
 
     KINDS = ("embed_ln", "bias_res_ln", "bias_gelu", "mask_scale_softmax", "bias_tanh", "mean_pool", "row_softmax",
-             "dense_gemm", "attention_gemm", "attention_fused", "classifier_head", "dense_split")
+             "dense_gemm", "attention_gemm", "attention_fused", "classifier_head", "dense_split",
+             "dense_qkv", "dense_attention_output", "dense_intermediate", "dense_output", "dense_pooler")
+    # a Dense launch is timed under its own kind when that kind is on and under "dense_gemm" otherwise
+    DENSE_KINDS = ("dense_qkv", "dense_attention_output", "dense_intermediate", "dense_output", "dense_pooler")
 
     def profile(self, kinds):
         """Switch per-kernel event timing on for the named kinds (empty = off)."""

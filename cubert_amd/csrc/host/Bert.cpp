@@ -292,7 +292,7 @@ void Bert<T>::forward(size_t batch_size) {
     bool tanh_pending = false;
     if (has_pooler_dense) {
         // first token of every sequence: the B rows are seq_length*hidden apart
-        Timed t(&profiler, Profiler::kDenseGemm, stream);
+        Timed t(&profiler, profiler.dense_kind(Profiler::kDensePooler), stream);
         cuBERT::blas_gemm(cublas, false, false, H, B, H, 1.f, pooler_kernel, H, _sequence_output, H * S, 0.f,
                           _pooled_output, H);
         tanh_pending = true;

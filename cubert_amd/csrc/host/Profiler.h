@@ -27,8 +27,18 @@ public:
         kAttentionFused = 9,
         kClassifierHead = 10,
         kDenseSplit = 11,  // fp32 rows written as two-term fp16 rows ahead of a Dense GEMM
-        kKinds = 12
+        // The Dense GEMMs one by one: a Dense launch is timed under its own kind when that kind is on, under
+        // kDenseGemm otherwise (so a caller sees either the sum or the parts, never the same launch twice).
+        kDenseQkv = 12,              // Q | K | V projection, [hidden] -> [3 * hidden]
+        kDenseAttentionOutput = 13,  // attention output, [hidden] -> [hidden]
+        kDenseIntermediate = 14,     // feed-forward up, [hidden] -> [intermediate]
+        kDenseOutput = 15,           // feed-forward down, [intermediate] -> [hidden]
+        kDensePooler = 16,           // BertPooler, [hidden] -> [hidden] on the first token of every sequence
+        kKinds = 17
     };
+
+    // The kind a Dense launch is timed under: its own when that is on, else the aggregate.
+    Kind dense_kind(Kind detail) const { return on(detail) ? detail : kDenseGemm; }
 
     ~Profiler() {
         for (auto &e : pool) {

@@ -276,9 +276,9 @@ bool Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *ma
 // otherwise it is left to the fused kernel that follows (which then reads the GEMM output once anyway).
 template <typename T>
 bool Transformer<T>::dense(int out_features, int tokens, int in_features, const T *kernel, const T *packed, const T *in,
-                           T *out, const T *bias, bool bias_in_gemm, bool gelu, int ld_out) {
+                           T *out, const T *bias, bool bias_in_gemm, bool gelu, Profiler::Kind kind, int ld_out) {
     void *stream = cuBERT::blas_get_stream(cublas);
-    Timed t(profiler, Profiler::kDenseGemm, stream);
+    Timed t(profiler, profiler != nullptr ? profiler->dense_kind(kind) : Profiler::kDenseGemm, stream);
     if (ld_out == 0) ld_out = out_features;
     // (the few-token kernel reads [in, out] kernels or its own copy of them, not transposed ones)
     if (tokens <= 32 && (packed != nullptr || (!transposed_kernels && gelu && dense_gelu_fits))) {
@@ -297,7 +297,7 @@ bool Transformer<T>::dense(int out_features, int tokens, int in_features, const 
 
 template <typename T>
 void Transformer<T>::dense_split(int out_features, int tokens, int in_features, const SplitKernel &kernel, const T *in,
-                                 T *out, const T *bias, int ld_out) {
+                                 T *out, const T *bias, Profiler::Kind kind, int ld_out) {
     if (ld_out == 0) ld_out = out_features;
     if constexpr (sizeof(T) == 4) {
         void *stream = cuBERT::blas_get_stream(cublas);
@@ -305,7 +305,7 @@ void Transformer<T>::dense_split(int out_features, int tokens, int in_features, 
             Timed t(profiler, Profiler::kDenseSplit, stream);
             cuBERT::split3(in, tokens, in_features, kTwoTermActivationScale, false, split_operand, stream);
         }
-        Timed t(profiler, Profiler::kDenseGemm, stream);
+        Timed t(profiler, profiler != nullptr ? profiler->dense_kind(kind) : Profiler::kDenseGemm, stream);
         cuBERT::blas_gemm_f16_f32(cublas, true, false, out_features, tokens, 3 * in_features,
                                   kernel.unscale / kTwoTermActivationScale,
                                   kernel.weights, 3 * in_features, split_operand, 3 * in_features, 0.f, out,
@@ -341,10 +341,10 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
                 // split_operand holds the two-term rows of the next Dense input whenever the kernel before it could
                 // write them itself (LayerNorm, GELU); otherwise dense_split makes them from the fp32 rows
                 dense_split(3 * H, M, H, w.qkv_split, operand_ready ? nullptr : layer_input, qkv_out, w.qkv_bias,
-                            (int) qkv_ld);
+                            Profiler::kDenseQkv, (int) qkv_ld);
                 const bool context_ready = attention(batch_size, qkv_out, attention_mask, split_operand);
                 dense_split(H, M, H, w.attention_output_split, context_ready ? nullptr : context_out, attention_output,
-                            nullptr);
+                            nullptr, Profiler::kDenseAttentionOutput);
                 {
                     Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
                     operand_ready = norm_writes_operand &&
@@ -358,14 +358,14 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
                     }
                 }
                 dense_split(I, M, H, w.intermediate_split, operand_ready ? nullptr : attention_output,
-                            intermediate_output, nullptr);
+                            intermediate_output, nullptr, Profiler::kDenseIntermediate);
                 {
                     // bias + GELU straight into the two-term rows the output Dense reads
                     Timed t(profiler, Profiler::kBiasGelu, stream);
                     cuBERT::bias_gelu_split3(intermediate_output, w.intermediate_bias, M, I, kTwoTermActivationScale,
                                              split_operand, stream);
                 }
-                dense_split(H, M, I, w.output_split, nullptr, out, nullptr);
+                dense_split(H, M, I, w.output_split, nullptr, out, nullptr, Profiler::kDenseOutput);
                 {
                     Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
                     operand_ready = norm_writes_operand &&
@@ -384,12 +384,14 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
         }
 
         // attention/self: row-major Y[M, N] = X[M, K] W[K, N] is the column-major gemm(N, M, K) on (W, X)
-        dense(3 * H, M, H, w.qkv_kernel, w.qkv_packed, layer_input, qkv_out, w.qkv_bias, true, false, (int) qkv_ld);
+        dense(3 * H, M, H, w.qkv_kernel, w.qkv_packed, layer_input, qkv_out, w.qkv_bias, true, false, Profiler::kDenseQkv,
+              (int) qkv_ld);
         attention(batch_size, qkv_out, attention_mask);
 
         // attention/output: dense, then bias + residual(layer input) + LayerNorm
         const bool ao_bias = dense(H, M, H, w.attention_output_kernel, w.attention_output_packed, context_out,
-                                   attention_output, w.attention_output_bias, false, false);
+                                   attention_output, w.attention_output_bias, false, false,
+                                   Profiler::kDenseAttentionOutput);
         {
             Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
             cuBERT::layer_norm_(layer_input, attention_output, M, H, ao_bias ? nullptr : w.attention_output_bias,
@@ -398,14 +400,14 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
 
         // intermediate: dense, then bias + GELU (one launch for all three at <= 32 tokens)
         if (!dense(I, M, H, w.intermediate_kernel, w.intermediate_packed, attention_output, intermediate_output,
-                   w.intermediate_bias, false, true)) {
+                   w.intermediate_bias, false, true, Profiler::kDenseIntermediate)) {
             Timed t(profiler, Profiler::kBiasGelu, stream);
             cuBERT::gelu(intermediate_output, w.intermediate_bias, M, I, stream);
         }
 
         // output: dense, then bias + residual(attention output) + LayerNorm
         const bool out_bias = dense(H, M, I, w.output_kernel, w.output_packed, intermediate_output, out, w.output_bias,
-                                    false, false);
+                                    false, false, Profiler::kDenseOutput);
         {
             Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
             cuBERT::layer_norm_(attention_output, out, M, H, out_bias ? nullptr : w.output_bias, w.output_norm_beta,

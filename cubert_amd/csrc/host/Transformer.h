@@ -95,11 +95,11 @@ private:
     // out[tokens, out_features] = in[tokens, in_features] * kernel (+ bias) (, GELU); returns whether bias and
     // activation were applied (false: the caller's fused kernel still has to).
     bool dense(int out_features, int tokens, int in_features, const T *kernel, const T *packed, const T *in, T *out,
-               const T *bias, bool bias_in_gemm, bool gelu, int ld_out = 0);
+               const T *bias, bool bias_in_gemm, bool gelu, Profiler::Kind kind, int ld_out = 0);
     // The same on the fp16 matrix cores from two-term operands (fp32 models only): `in` is split into
     // split_operand first, or, when null, split_operand already holds the [hi | hi | lo] rows.  `bias` may be null.
     void dense_split(int out_features, int tokens, int in_features, const SplitKernel &kernel, const T *in, T *out,
-                     const T *bias, int ld_out = 0);
+                     const T *bias, Profiler::Kind kind, int ld_out = 0);
 
     void *cublas;
     Profiler *profiler = nullptr;

@@ -132,9 +132,10 @@ int cubert_bert_output(void *bert, int dtype, int batch_size, cuBERT_Output *out
 int cubert_bert_compute_resident(void *bert, int dtype, int batch_size);
 /* Per-kernel timing with stream events: bit k of `kinds` switches kind k on (0 embed+LN, 1 bias+residual+LN,
  * 2 bias+GELU, 3 mask+scale+softmax, 4 bias+tanh, 5 mean pool, 6 row softmax, 7 dense GEMM, 8 attention GEMM,
- * 9 fused attention, 10 classifier head).  cubert_bert_profile_read synchronises, adds the elapsed milliseconds and
- * launch counts seen since the last read to total_ms[kind] / count[kind] (arrays of n_kinds >= 12 entries) and
- * forgets them. */
+ * 9 fused attention, 10 classifier head, 11 two-term operand rows; 12-16 the Dense GEMMs one by one: Q|K|V,
+ * attention output, intermediate, output, pooler -- a Dense launch is timed under its own kind when that is on and
+ * under kind 7 otherwise).  cubert_bert_profile_read synchronises, adds the elapsed milliseconds and launch counts
+ * seen since the last read to total_ms[kind] / count[kind] (arrays of n_kinds >= 17 entries) and forgets them. */
 int cubert_bert_profile(void *bert, int dtype, unsigned kinds);
 int cubert_bert_profile_read(void *bert, int dtype, double *total_ms, int *count, int n_kinds);
 /* The HIP stream the model's work is enqueued on. */
