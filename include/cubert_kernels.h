@@ -347,7 +347,16 @@ int cubert_gemm_strided_batch_f16(void *handle, int transA, int transB, int M, i
  * transposes are shared.  fp32 accumulation; with beta = 0 the C matrices are not read.  Runs on the handle's
  * stream, asynchronously.  This is the interface of the reference's attention contractions (Att_Q_K / Att_QK_V
  * build one pointer per (batch, head), src/cuBERT/op_att/BatchMatMul.cpp:31-38,57-68,103-110,129-140); the host
- * classes here use cubert_attention_* instead, which is the fast path.
+ * classes here use cubert_attention_* instead, which is the fast path.  This entry point is the compatibility
+ * path for a host program that keeps the reference's BatchMatMul classes: shapes whose M, N and K are multiples of
+ * 32 run on the matrix cores (a wavefront per 32 x 32 tile of C), any other shape on plain fused multiply-adds.
+ * What it costs, measured on one MI355X on the QK^T contraction of 1536 (batch, head) problems of head size 64,
+ * microseconds per launch, this entry point / cubert_attention_scores_* on the same operands:
+ *   fp32  seq 32:  8.3 / 10.0    seq 128:  73.6 / 128.3
+ *   fp16  seq 32:  4.9 /  4.5    seq 128:  40.5 /  17.3
+ * (before the matrix-core kernel: 21.3, 114.3, 19.4 and 96.8).  Either way a host that goes through this interface
+ * writes the [batch, heads, seq, seq] tensor to memory and reads it back twice, which cubert_attention_fused_* does
+ * not: one launch of 12.7 us (fp32, seq 32) instead of three.
  * replaces: blas_gemm_batch<T>, reference src/cuBERT/common.h:70-80 (src/cuBERT/common.cpp:261-298,375-396). */
 int cubert_gemm_batch_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha,
                           const float *const *A_array, int lda, const float *const *B_array, int ldb, float beta,

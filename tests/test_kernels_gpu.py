@@ -200,11 +200,15 @@ def test_batch_matmul_reference_vectors_pointer_arrays(K, case):
 @pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
 @pytest.mark.parametrize("M,N,K_,batch", [(32, 32, 64, 24), (64, 128, 128, 5), (70, 65, 19, 3), (1, 1, 1, 2),
                                           (128, 128, 64, 7), (5, 200, 33, 4)])
-def test_gemm_batch_against_oracle_sgemm(K, name, ta, tb, M, N, K_, batch):
-    """blas_gemm_batch (arrays of pointers, column-major, all transposes, alpha / beta, padded leading dimensions,
-    tile edges) against the oracle's sgemm problem by problem."""
+@pytest.mark.parametrize("padded", [True, False])
+def test_gemm_batch_against_oracle_sgemm(K, name, ta, tb, M, N, K_, batch, padded):
+    """blas_gemm_batch (arrays of pointers, column-major, all transposes, alpha / beta, tile edges) against the
+    oracle's sgemm problem by problem; leading dimensions padded by odd amounts (element accesses) and exact (the
+    16-byte accesses of the matrix-core kernel that shapes of whole 32 x 32 x 32 tiles take)."""
     rng = np.random.default_rng(M * 31 + N * 7 + K_ + batch + 2 * ta + tb)
-    lda, ldb, ldc = (K_ if ta else M) + 3, (N if tb else K_) + 2, M + 1
+    lda, ldb, ldc = (K_ if ta else M), (N if tb else K_), M
+    if padded:
+        lda, ldb, ldc = lda + 3, ldb + 2, ldc + 1
     a_cols, b_cols = (M if ta else K_), (K_ if tb else N)
     As = [q(rng.normal(0, 1, lda * a_cols), name) for _ in range(batch)]
     Bs = [q(rng.normal(0, 1, ldb * b_cols), name) for _ in range(batch)]
