@@ -101,10 +101,10 @@ SIGNATURES = {
     "cubert_gemm_skinny_noalloc_f32": (ci, [vp, ci, ci, ci, cf, vp, ci, vp, ci, vp, ci, vp, ci]),
     "cubert_gemm_skinny_packed_elements": (ctypes.c_size_t, [ci, ci]),
     "cubert_gemm_f16_f32": (ci, [vp, ci, ci, ci, ci, ci, cf, vp, ci, vp, ci, cf, vp, ci, vp]),
-    "cubert_split3_f32": (ci, [vp, ci, ci, cf, ci, vp, vp]),
-    "cubert_bias_gelu_split3_f32": (ci, [vp, vp, ci, ci, cf, vp, vp]),
-    "cubert_attention_fused_split3_f32": (ci, [vp, vp, vp, ci, vp, cf, vp, cf, ci, ci, ci, ci, vp]),
-    "cubert_bias_res_ln_split3_f32": (ci, [vp, vp, vp, vp, vp, ci, ci, cf, vp, vp]),
+    "cubert_split3_f32": (ci, [vp, ci, ci, cf, ci, vp, vp, vp]),
+    "cubert_bias_gelu_split3_f32": (ci, [vp, vp, ci, ci, cf, vp, vp, vp]),
+    "cubert_attention_fused_split3_f32": (ci, [vp, vp, vp, ci, vp, cf, vp, cf, ci, ci, ci, ci, vp, vp]),
+    "cubert_bias_res_ln_split3_f32": (ci, [vp, vp, vp, vp, vp, ci, ci, cf, vp, vp, vp]),
     "cubert_blas_create": (vp, []),
     "cubert_blas_destroy": (ci, [vp]),
     "cubert_blas_set_stream": (ci, [vp, vp]),

@@ -206,6 +206,7 @@ void Bert<T>::_pre_compute(size_t batch_size) {
     segment_ids_buf = reinterpret_cast<int8_t *>(input_block + segments_at);
     forward(batch_size);
     synchronize();
+    (void) transformer->two_term_overflowed();  // what the made-up inputs did says nothing about a request
     input_ids_buf = nullptr, input_mask_buf = nullptr, segment_ids_buf = nullptr;  // no request is resident
 }
 
@@ -220,6 +221,12 @@ void Bert<T>::synchronize() {
 // page-locked block first and reach the caller's array after the stream has drained.
 template <typename T>
 void Bert<T>::fetch(void *dst, const void *src, size_t bytes) {
+    requested.push_back(RequestedOutput{dst, src, bytes});
+    enqueue_fetch(dst, src, bytes);
+}
+
+template <typename T>
+void Bert<T>::enqueue_fetch(void *dst, const void *src, size_t bytes) {
     const size_t at = round_up_16(staged_bytes);
     if (output_staging != nullptr && at + bytes <= kOutputStagingBytes) {
         cuBERT::memcpyAsync(output_staging + at, src, bytes, 2, stream);
@@ -233,9 +240,22 @@ void Bert<T>::fetch(void *dst, const void *src, size_t bytes) {
 template <typename T>
 void Bert<T>::finish_outputs() {
     synchronize();
+    // An fp32 model in the two-term fp16 Dense form (opt-in): an activation beyond what two fp16 terms can hold
+    // raised a flag while the request ran.  Its results are not to be trusted: the same request, whose inputs are
+    // still on the device, runs again on the fp32 GEMMs, and the copies this call asked for are made again.
+    if (transformer != nullptr && transformer->two_term_overflowed() && last_batch > 0 && input_ids_buf != nullptr) {
+        transformer->use_fp32_dense_once();
+        forward(last_batch);
+        staged.clear();
+        staged_bytes = 0;
+        for (const RequestedOutput &o : requested) enqueue_fetch(o.dst, o.src, o.bytes);
+        synchronize();
+        (void) transformer->two_term_overflowed();  // (the fp32 pass writes no two-term rows; nothing to clear)
+    }
     for (const StagedOutput &o : staged) std::memcpy(o.dst, output_staging + o.offset, o.bytes);
     staged.clear();
     staged_bytes = 0;
+    requested.clear();
 }
 
 template <typename T>
@@ -275,6 +295,7 @@ void Bert<T>::compute_resident(size_t batch_size) {
 
 template <typename T>
 void Bert<T>::forward(size_t batch_size) {
+    last_batch = batch_size;
     const int B = (int) batch_size, S = (int) seq_length, H = (int) hidden_size, L = (int) num_labels;
 
     // bert/embeddings

@@ -78,7 +78,8 @@ public:
 private:
     void forward(size_t batch_size);
     void synchronize();       // drains the stream
-    void fetch(void *dst, const void *src, size_t bytes);  // queue one device-to-host output copy
+    void fetch(void *dst, const void *src, size_t bytes);  // queue one device-to-host output copy and remember it
+    void enqueue_fetch(void *dst, const void *src, size_t bytes);
     void finish_outputs();    // drain the stream and hand staged outputs to the caller's arrays
     void release() noexcept;  // everything the constructor acquired so far (also run when it throws)
     void layout_weights(size_t vocab_size, size_t type_vocab_size);
@@ -116,6 +117,14 @@ private:
     unsigned char *output_staging = nullptr;
     std::vector<StagedOutput> staged;
     size_t staged_bytes = 0;
+    // every copy an output call has asked for, so that the call can be repeated after the request was recomputed
+    struct RequestedOutput {
+        void *dst;
+        const void *src;
+        size_t bytes;
+    };
+    std::vector<RequestedOutput> requested;
+    size_t last_batch = 0;               // batch size of the forward pass whose results the buffers hold
     bool input_copy_pending = false;     // a copy out of input_staging was queued and the stream not drained since
     int *input_ids_buf;
     int8_t *input_mask_buf;

@@ -52,6 +52,12 @@ Transformer<T>::Transformer(void *cublas, const std::string &var_prefix,
     split_dense = sizeof(T) == 4 && dense_mode != nullptr && std::string(dense_mode) == "f16x3" &&
                   max_batch_size * seq_length >= kTwoTermMinTokens;
 
+    if (split_dense) {
+        split_overflow = static_cast<int *>(cubert_malloc_host(64));
+        if (split_overflow == nullptr) throw std::runtime_error("no page-locked host memory for the two-term overflow flag");
+        *split_overflow = 0;
+    }
+
     // Weight names as the reference resolves them (Transformer.cpp:54-101, AttentionSelf.cpp:27-44);
     // a missing name throws std::out_of_range from unordered_map::at, as it does there.
     layout_weights();
@@ -83,7 +89,9 @@ Transformer<T>::Transformer(void *cublas, const std::string &var_prefix,
                 }
                 split.unscale = std::ldexp(1.f, -exponent);
                 cuBERT::transpose(dst, (int) in, (int) out, staging, stream);
-                cuBERT::split3(staging, (int) out, (int) in, std::ldexp(1.f, exponent), true, split.weights, stream);
+                // (weights are scaled into [512, 1024): no overflow flag needed on this side)
+                cuBERT::split3(staging, (int) out, (int) in, std::ldexp(1.f, exponent), true, split.weights, nullptr,
+                               stream);
                 cuBERT::cuda_stream_synchronize(stream);
             }
         }
@@ -125,6 +133,18 @@ Transformer<T>::Transformer(void *cublas, const std::string &var_prefix,
     layout_buffers();
     buffers.allocate();
     layout_buffers();
+}
+
+template <typename T>
+Transformer<T>::~Transformer() {
+    cubert_free_host(split_overflow);  // null is accepted
+}
+
+template <typename T>
+bool Transformer<T>::two_term_overflowed() {
+    if (split_overflow == nullptr || *static_cast<volatile int *>(split_overflow) == 0) return false;
+    *split_overflow = 0;
+    return true;
 }
 
 template <typename T>
@@ -224,7 +244,7 @@ bool Transformer<T>::attention(size_t batch_size, const T *qkv, const int8_t *ma
         if constexpr (sizeof(T) == 4) {
             if (split_context != nullptr &&
                 cuBERT::attention_fused_split3(Q, K, V, ld, mask, kTwoTermActivationScale, split_context, alpha, B, A, S,
-                                               d, stream)) {
+                                               d, split_overflow, stream)) {
                 return true;
             }
         }
@@ -303,7 +323,8 @@ void Transformer<T>::dense_split(int out_features, int tokens, int in_features, 
         void *stream = cuBERT::blas_get_stream(cublas);
         if (in != nullptr) {
             Timed t(profiler, Profiler::kDenseSplit, stream);
-            cuBERT::split3(in, tokens, in_features, kTwoTermActivationScale, false, split_operand, stream);
+            cuBERT::split3(in, tokens, in_features, kTwoTermActivationScale, false, split_operand, split_overflow,
+                           stream);
         }
         Timed t(profiler, profiler != nullptr ? profiler->dense_kind(kind) : Profiler::kDenseGemm, stream);
         cuBERT::blas_gemm_f16_f32(cublas, true, false, out_features, tokens, 3 * in_features,
@@ -323,7 +344,8 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
 
     // (small requests are bound by the pass over the weights, which are 6 bytes per parameter in two-term form and 4
     // in fp32: they keep the fp32 kernels)
-    const bool split = split_dense && (size_t) M >= kTwoTermMinTokens;
+    const bool split = split_dense && (size_t) M >= kTwoTermMinTokens && !fp32_dense_once;
+    fp32_dense_once = false;
     bool operand_ready = false;
 
     // long sequences: the attention kernels take the sequences longest first (the mask is the same for every layer)
@@ -350,7 +372,8 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
                     operand_ready = norm_writes_operand &&
                                     cuBERT::layer_norm_split3(layer_input, attention_output, M, H, w.attention_output_bias,
                                                               w.attention_norm_beta, w.attention_norm_gamma,
-                                                              kTwoTermActivationScale, split_operand, stream);
+                                                              kTwoTermActivationScale, split_operand, split_overflow,
+                                                              stream);
                     if (!operand_ready) {
                         norm_writes_operand = false;  // the hidden size is fixed per model: do not ask again
                         cuBERT::layer_norm_(layer_input, attention_output, M, H, w.attention_output_bias,
@@ -363,7 +386,7 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
                     // bias + GELU straight into the two-term rows the output Dense reads
                     Timed t(profiler, Profiler::kBiasGelu, stream);
                     cuBERT::bias_gelu_split3(intermediate_output, w.intermediate_bias, M, I, kTwoTermActivationScale,
-                                             split_operand, stream);
+                                             split_operand, split_overflow, stream);
                 }
                 dense_split(H, M, I, w.output_split, nullptr, out, nullptr, Profiler::kDenseOutput);
                 {
@@ -371,7 +394,8 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
                     operand_ready = norm_writes_operand &&
                                     cuBERT::layer_norm_split3(attention_output, out, M, H, w.output_bias,
                                                               w.output_norm_beta, w.output_norm_gamma,
-                                                              kTwoTermActivationScale, split_operand, stream);
+                                                              kTwoTermActivationScale, split_operand, split_overflow,
+                                                              stream);
                     if (!operand_ready) {
                         norm_writes_operand = false;
                         cuBERT::layer_norm_(attention_output, out, M, H, w.output_bias, w.output_norm_beta,

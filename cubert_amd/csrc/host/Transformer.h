@@ -44,7 +44,10 @@ public:
                          size_t max_batch_size, size_t seq_length, size_t hidden_size, size_t num_hidden_layers,
                          size_t num_attention_heads, size_t intermediate_size);
 
-    virtual ~Transformer() = default;
+    virtual ~Transformer();
+
+    Transformer(const Transformer &) = delete;
+    Transformer &operator=(const Transformer &) = delete;
 
     T *compute(size_t batch_size, T *input_gpu, int8_t *attention_mask);
 
@@ -57,6 +60,14 @@ public:
 
     // Optional per-kernel timing (owned by the caller; null = off).
     void set_profiler(Profiler *p) { profiler = p; }
+
+    // Two-term fp16 Dense form only (CUBERT_FP32_DENSE=f16x3).  An activation beyond the fp16 range (|16 x| > 65504)
+    // cannot be written as two fp16 terms; the kernels that write two-term rows then raise a flag instead of
+    // handing a clamped operand to the GEMM in silence.  Once the stream has drained, two_term_overflowed() says
+    // whether any request since the last call raised it (and clears it); the caller then runs the request again
+    // after use_fp32_dense_once(), which makes the next _in_compute take the fp32 GEMMs whatever its size.
+    bool two_term_overflowed();
+    void use_fp32_dense_once() { fp32_dense_once = true; }
 
 private:
     // A Dense kernel for the two-term fp16 form: rows [hi | lo | hi] of scale * W^T, [out, 3 * in]; unscale = 1 / scale
@@ -107,6 +118,8 @@ private:
     bool keep_packed = false;          // Dense kernels are also kept in the few-token kernel's order
     bool transposed_kernels = false;   // Dense kernels are stored [out, in] instead of [in, out] (half precision)
     bool split_dense = false;          // fp32 model with Dense layers in the two-term fp16 form (opt-in)
+    bool fp32_dense_once = false;      // the next request takes the fp32 GEMMs (set after a two-term overflow)
+    int *split_overflow = nullptr;     // page-locked host word the two-term kernels set to 1 on overflow (split_dense)
     bool norm_writes_operand = true;   // cleared when the LayerNorm that also writes two-term rows declines the hidden size
     bool fused_attention_fits = true;  // cleared when the one-launch attention kernel declines this model's shape
     size_t max_batch_size, seq_length, hidden_size, num_hidden_layers, num_attention_heads, intermediate_size;

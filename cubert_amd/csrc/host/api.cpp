@@ -162,6 +162,12 @@ void transformer_run(const char *prefix, int n, const char *const *names, const 
         T *out_gpu = transformer.compute(batch, in_gpu, mask_gpu);
         cuBERT::memcpyAsync(output, out_gpu, count * sizeof(T), 2, stream);
         cuBERT::cuda_stream_synchronize(stream);
+        if (transformer.two_term_overflowed()) {  // opt-in two-term fp16 Dense form: an activation did not fit, again in fp32
+            transformer.use_fp32_dense_once();
+            out_gpu = transformer.compute(batch, in_gpu, mask_gpu);
+            cuBERT::memcpyAsync(output, out_gpu, count * sizeof(T), 2, stream);
+            cuBERT::cuda_stream_synchronize(stream);
+        }
         cuBERT::free(mask_gpu);
         cuBERT::free(in_gpu);
     }

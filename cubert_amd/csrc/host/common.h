@@ -115,14 +115,17 @@ inline void blas_gemm_f16_f32(void *handle, bool TransA, bool TransB, int M, int
                               const float *bias = nullptr) {
     CUBERT_CHECK(cubert_gemm_f16_f32(handle, TransA, TransB, M, N, K, alpha, h(A), lda, h(B), ldb, beta, C, ldc, bias));
 }
-inline void split3(const float *in, int rows, int width, float scale, bool lo_in_middle, half *out, void *stream) {
-    CUBERT_CHECK(cubert_split3_f32(in, rows, width, scale, lo_in_middle, h(out), stream));
+// (`overflow` in this and the next three: where 1 is stored when a value did not fit its two terms; may be null)
+inline void split3(const float *in, int rows, int width, float scale, bool lo_in_middle, half *out, int *overflow,
+                   void *stream) {
+    CUBERT_CHECK(cubert_split3_f32(in, rows, width, scale, lo_in_middle, h(out), overflow, stream));
 }
 // false: the shape is not one the fused kernel takes (the caller runs layer_norm_ and split3)
 inline bool layer_norm_split3(const float *in, float *inout, int rows, int channels, const float *bias,
-                              const float *beta, const float *gamma, float scale, half *split_out, void *stream) {
+                              const float *beta, const float *gamma, float scale, half *split_out, int *overflow,
+                              void *stream) {
     const int rc = cubert_bias_res_ln_split3_f32(inout, in, bias, beta, gamma, rows, channels, scale, h(split_out),
-                                                 stream);
+                                                 overflow, stream);
     if (rc == CUBERT_UNSUPPORTED) return false;
     CUBERT_CHECK(rc);
     return true;
@@ -130,16 +133,16 @@ inline bool layer_norm_split3(const float *in, float *inout, int rows, int chann
 // the one-launch attention core with its context in two-term rows; false when the shape is not taken
 inline bool attention_fused_split3(const float *q, const float *k, const float *v, int ld, const int8_t *mask,
                                    float scale, half *split_ctx, float alpha, int batch, int heads, int seq,
-                                   int head_size, void *stream) {
+                                   int head_size, int *overflow, void *stream) {
     const int rc = cubert_attention_fused_split3_f32(q, k, v, ld, mask, scale, h(split_ctx), alpha, batch, heads, seq,
-                                                     head_size, stream);
+                                                     head_size, overflow, stream);
     if (rc == CUBERT_UNSUPPORTED) return false;
     CUBERT_CHECK(rc);
     return true;
 }
 inline void bias_gelu_split3(const float *in, const float *bias, int rows, int width, float scale, half *out,
-                             void *stream) {
-    CUBERT_CHECK(cubert_bias_gelu_split3_f32(in, bias, rows, width, scale, h(out), stream));
+                             int *overflow, void *stream) {
+    CUBERT_CHECK(cubert_bias_gelu_split3_f32(in, bias, rows, width, scale, h(out), overflow, stream));
 }
 
 inline void transpose(const float *in, int rows, int cols, float *out, void *stream) {

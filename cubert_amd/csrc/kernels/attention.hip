@@ -60,25 +60,33 @@ struct Mma<float> {
 // Accumulator register i of lane (r = lane % 32, hh = lane / 32) is element (row, col) of the tile:
 __device__ __forceinline__ int acc_row(int i, int hh) { return (i >> 2) * 8 + hh * 4 + (i & 3); }
 
-// One element of the attention context.  split_width = 0: ctx[row, col] in the storage type.  split_width = W > 0
+// Where the context goes when it is wanted in two-term form (fp32 models whose Dense layers run on the fp16 matrix
+// cores): width = 0 means the ordinary store.
+struct SplitOut {
+    int width = 0;            // halves per part of a row [hi | hi | lo]
+    float scale = 1.f;        // applied before the value is taken apart
+    int *overflow = nullptr;  // set to 1 when a scaled value is outside the fp16 range (or not a number); may be null
+};
+
+// One element of the attention context.  split.width = 0: ctx[row, col] in the storage type.  split.width = W > 0
 // (fp32 only): `ctx` is really a buffer of halves with rows [hi | hi | lo] of W each, the two-term form of
-// split_scale * v that the Dense GEMM on the fp16 matrix cores reads (hi = fp16(.), lo = fp16(. - hi), clamped to
-// the fp16 range).
+// split.scale * v that the Dense GEMM on the fp16 matrix cores reads (hi = fp16(.), lo = fp16(. - hi), clamped to
+// the fp16 range; a value that had to be clamped raises split.overflow, and the caller recomputes in fp32).
 // (SPLIT is a compile-time choice so that the plain kernels are exactly what they were without it.)
 template <typename T, bool SPLIT>
-__device__ __forceinline__ void store_context(T *ctx, int ld_ctx, size_t row, int col, float v, int split_width,
-                                              float split_scale) {
+__device__ __forceinline__ void store_context(T *ctx, int ld_ctx, size_t row, int col, float v, const SplitOut &split) {
     if constexpr (SPLIT) {
         // v as the plain kernel would store it: rounded to fp32 before it is taken apart (without this the compiler
         // fuses a product that made v into the subtraction below, and lo would belong to the unrounded value)
         asm volatile("" : "+v"(v));
-        v *= split_scale;
-        half_t *p = reinterpret_cast<half_t *>(ctx) + row * 3 * split_width + col;
+        v *= split.scale;
+        half_t *p = reinterpret_cast<half_t *>(ctx) + row * 3 * split.width + col;
         half_t hi, lo;
         split_two_terms(v, hi, lo);
+        if (two_term_overflow(v) && split.overflow != nullptr) *split.overflow = 1;
         p[0] = hi;
-        p[split_width] = hi;
-        p[2 * split_width] = lo;
+        p[split.width] = hi;
+        p[2 * split.width] = lo;
     } else {
         ctx[row * ld_ctx + col] = from_f32<T>(v);
     }
@@ -330,7 +338,7 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
                                                                      const T *__restrict__ v, int ld,
                                                                      const int8_t *__restrict__ mask,
                                                                      T *__restrict__ ctx, int ld_ctx, float alpha,
-                                                                     int heads, int split_width, float split_scale) {
+                                                                     int heads, SplitOut split) {
     constexpr int V = Mma<T>::kVec;
     constexpr int kSteps = D / 2 / V;
     constexpr int kColTiles = D / 32;
@@ -467,8 +475,7 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_kernel(const T *__
     for (int jt = 0; jt < kColTiles; ++jt) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            store_context<T, SPLIT>(ctx, ld_ctx, first_row + acc_row(i, hh), h * D + jt * 32 + r, out[jt][i], split_width,
-                                    split_scale);
+            store_context<T, SPLIT>(ctx, ld_ctx, first_row + acc_row(i, hh), h * D + jt * 32 + r, out[jt][i], split);
         }
     }
 }
@@ -740,7 +747,7 @@ __global__ __launch_bounds__(4 * kWave) void attention_small_kernel(const T *__r
                                                                     const T *__restrict__ v, int ld,
                                                                     const int8_t *__restrict__ mask,
                                                                     T *__restrict__ ctx, int ld_ctx, float alpha,
-                                                                    int heads, int split_width, float split_scale) {
+                                                                    int heads, SplitOut split) {
     constexpr int D = 64, S = 32;
     constexpr int V = Mma<T>::kVec;
     constexpr int kSteps = D / 8 / V;  // operand vectors per lane and contraction: a quarter of D over two lane halves
@@ -828,7 +835,7 @@ __global__ __launch_bounds__(4 * kWave) void attention_small_kernel(const T *__r
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             store_context<T, SPLIT>(ctx, ld_ctx, (size_t) row0 + acc_row(i, hh), h * D + jt * 32 + r,
-                             out[i] + s_part[jt][i * kWave + lane], split_width, split_scale);
+                             out[i] + s_part[jt][i * kWave + lane], split);
         }
     }
 }
@@ -853,8 +860,7 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
                                                                const T *__restrict__ v, int ld,
                                                                const int8_t *__restrict__ mask, T *__restrict__ ctx,
                                                                int ld_ctx, float alpha, int heads, int seq,
-                                                               int skip_masked_tiles, int split_width,
-                                                               float split_scale, const int *__restrict__ order) {
+                                                               int skip_masked_tiles, SplitOut split, const int *__restrict__ order) {
     constexpr int V = Mma<T>::kVec;
     constexpr int kSteps = D / 2 / V;
     constexpr int kColTiles = D / 32;
@@ -1051,7 +1057,7 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 store_context<T, SPLIT>(ctx, ld_ctx, first_row + acc_row(g * 4 + e, hh), h * D + jt * 32 + r,
-                                 out[jt][g * 4 + e] * fr.v[e], split_width, split_scale);
+                                 out[jt][g * 4 + e] * fr.v[e], split);
             }
         }
     }
@@ -1069,7 +1075,7 @@ __global__ __launch_bounds__(1024) void attention_flash_kernel(const T *__restri
 template <typename T, int D, bool SPLIT>
 __global__ __launch_bounds__(1024) void attention_flash_grouped_kernel(
     const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, int ld, const int8_t *__restrict__ mask,
-    T *__restrict__ ctx, int ld_ctx, float alpha, int heads, int skip_masked_tiles, int split_width, float split_scale,
+    T *__restrict__ ctx, int ld_ctx, float alpha, int heads, int skip_masked_tiles, SplitOut split,
     const int *__restrict__ order) {
     constexpr int V = Mma<T>::kVec;
     constexpr int kSteps = D / 2 / V;
@@ -1285,7 +1291,7 @@ __global__ __launch_bounds__(1024) void attention_flash_grouped_kernel(
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 store_context<T, SPLIT>(ctx, ld_ctx, first_row + acc_row(g * 4 + e, hh), h * D + jt * 32 + r,
-                                        out[jt][g * 4 + e] * fr.v[e], split_width, split_scale);
+                                        out[jt][g * 4 + e] * fr.v[e], split);
             }
         }
     }
@@ -1438,21 +1444,21 @@ int attention_context(const T *probs, const T *v, int ld, T *ctx, int ld_ctx, in
 
 template <typename T, int D, int KT>
 int launch_fused_kt(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
-                    int batch, int heads, int split_width, float split_scale, hipStream_t s) {
+                    int batch, int heads, SplitOut split, hipStream_t s) {
     constexpr size_t lds = fused_lds_bytes<T, D, KT>();
     if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
     if constexpr (sizeof(T) == 4) {
-        if (split_width > 0) {
+        if (split.width > 0) {
             auto kernel = attention_fused_kernel<T, D, KT, true>;
             if (lds > 48 * 1024) {
                 static std::atomic<unsigned long long> raised{0};  // per instantiation
                 if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
             }
             return launch_lds(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask,
-                                  ctx, ld_ctx, alpha, heads, split_width, split_scale);
+                                  ctx, ld_ctx, alpha, heads, split);
         }
     }
-    if (split_width > 0) return CUBERT_UNSUPPORTED;
+    if (split.width > 0) return CUBERT_UNSUPPORTED;
     if constexpr (sizeof(T) == 2) {
         // CUBERT_ATTENTION_KERNEL=general / lean in the environment forces one of the two; by default the lean kernel
         // runs where the grid fills the chip several times over (measured at 128 keys, head size 64: 4096 workgroups
@@ -1480,47 +1486,43 @@ int launch_fused_kt(const T *q, const T *k, const T *v, int ld, const int8_t *ma
         if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
     }
     return launch_lds(kernel, dim3(batch * heads), dim3(KT * kWave), (unsigned) lds, s, q, k, v, ld, mask, ctx,
-                          ld_ctx, alpha, heads, split_width, split_scale);
+                          ld_ctx, alpha, heads, split);
 }
 
 template <typename T, int D>
 int launch_fused(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
-                 int batch, int heads, int seq, int split_width, float split_scale, hipStream_t s) {
+                 int batch, int heads, int seq, SplitOut split, hipStream_t s) {
     if constexpr (D == 64) {
         // split each problem over four wavefronts: a quarter of the dependent matrix instructions per wavefront
         // (12 problems 5.3 -> 4.7 us, 1536 problems 15.95 -> 15.0 us; not measured beyond)
         if (seq == 32 && batch * heads <= 2048 && (mask == nullptr || is_aligned(mask, 4))) {
             if constexpr (sizeof(T) == 4) {
-                if (split_width > 0) {
+                if (split.width > 0) {
                     return launch_lds(attention_small_kernel<T, true>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q,
-                                          k, v, ld, mask, ctx, ld_ctx, alpha, heads, split_width, split_scale);
+                                          k, v, ld, mask, ctx, ld_ctx, alpha, heads, split);
                 }
             }
-            if (split_width > 0) return CUBERT_UNSUPPORTED;
+            if (split.width > 0) return CUBERT_UNSUPPORTED;
             return launch_lds(attention_small_kernel<T, false>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q, k, v,
-                                  ld, mask, ctx, ld_ctx, alpha, heads, split_width, split_scale);
+                                  ld, mask, ctx, ld_ctx, alpha, heads, split);
         }
     }
     switch (seq / 32) {
         case 1:
-            return launch_fused_kt<T, D, 1>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width,
-                                             split_scale, s);
+            return launch_fused_kt<T, D, 1>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split, s);
         case 2:
-            return launch_fused_kt<T, D, 2>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width,
-                                             split_scale, s);
+            return launch_fused_kt<T, D, 2>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split, s);
         case 3:
-            return launch_fused_kt<T, D, 3>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width,
-                                             split_scale, s);
+            return launch_fused_kt<T, D, 3>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split, s);
         case 4:
-            return launch_fused_kt<T, D, 4>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split_width,
-                                             split_scale, s);
+            return launch_fused_kt<T, D, 4>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, split, s);
         default: return CUBERT_UNSUPPORTED;
     }
 }
 
 template <typename T, int D>
 int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
-                 int batch, int heads, int seq, int split_width, float split_scale, const int *order, hipStream_t s) {
+                 int batch, int heads, int seq, SplitOut split, const int *order, hipStream_t s) {
     constexpr int V = 16 / sizeof(T);
     if (seq > 512) return CUBERT_UNSUPPORTED;  // a workgroup has at most 16 wavefronts
     const size_t lds = (size_t) seq * (D + V) * sizeof(T) + (size_t) D * (seq + V) * sizeof(T) +
@@ -1532,39 +1534,38 @@ int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask,
         const size_t grouped_lds = ((size_t) G * 32 * (D + V) + (size_t) D * (G * 32 + V)) * sizeof(T) +
                                    ((size_t) seq + 16 * 32) * sizeof(float);
         if constexpr (sizeof(T) == 4) {
-            if (split_width > 0) {
+            if (split.width > 0) {
                 return launch_lds(attention_flash_grouped_kernel<T, D, true>, dim3(batch * heads), dim3(1024),
                                       (unsigned) grouped_lds, s, q, k, v, ld, mask, ctx, ld_ctx, alpha, heads,
-                                      skip_masked_tiles, split_width, split_scale, order);
+                                      skip_masked_tiles, split, order);
             }
         }
-        if (split_width > 0) return CUBERT_UNSUPPORTED;
+        if (split.width > 0) return CUBERT_UNSUPPORTED;
         return launch_lds(attention_flash_grouped_kernel<T, D, false>, dim3(batch * heads), dim3(1024),
                               (unsigned) grouped_lds, s, q, k, v, ld, mask, ctx, ld_ctx, alpha, heads, skip_masked_tiles,
-                              split_width, split_scale, order);
+                              split, order);
     }
     if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
     if constexpr (sizeof(T) == 4) {
-        if (split_width > 0) {
+        if (split.width > 0) {
             auto kernel = attention_flash_kernel<T, D, true>;
             static std::atomic<unsigned long long> raised{0};  // per instantiation
             if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
             return launch_lds(kernel, dim3(batch * heads), dim3(seq / 32 * kWave), (unsigned) lds, s, q, k, v, ld,
-                                  mask, ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles, split_width, split_scale, order);
+                                  mask, ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles, split, order);
         }
     }
-    if (split_width > 0) return CUBERT_UNSUPPORTED;
+    if (split.width > 0) return CUBERT_UNSUPPORTED;
     auto kernel = attention_flash_kernel<T, D, false>;
     static std::atomic<unsigned long long> raised{0};  // per instantiation
     if (!allow_large_lds(kernel, raised)) return CUBERT_UNSUPPORTED;
     return launch_lds(kernel, dim3(batch * heads), dim3(seq / 32 * kWave), (unsigned) lds, s, q, k, v, ld, mask,
-                          ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles, split_width, split_scale, order);
+                          ctx, ld_ctx, alpha, heads, seq, skip_masked_tiles, split, order);
 }
 
 template <typename T>
 int attention_fused(const T *q, const T *k, const T *v, int ld, const int8_t *mask, T *ctx, int ld_ctx, float alpha,
-                    int batch, int heads, int seq, int head_size, void *stream, int split_width = 0,
-                    float split_scale = 1.f, const int *order = nullptr) {
+                    int batch, int heads, int seq, int head_size, void *stream, SplitOut split = SplitOut(), const int *order = nullptr) {
     if (batch == 0 || heads == 0 || seq == 0) return 0;
     if (!q || !k || !v || !ctx || batch < 0 || heads < 0 || seq < 0 || head_size <= 0) return CUBERT_BAD_ARGUMENT;
     if (ld < heads * head_size) return CUBERT_BAD_ARGUMENT;
@@ -1575,23 +1576,21 @@ int attention_fused(const T *q, const T *k, const T *v, int ld, const int8_t *ma
     if (seq > 128) {
         switch (head_size) {
             case 32:
-                return launch_flash<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width,
-                                           split_scale, order, s);
+                return launch_flash<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split, order, s);
             case 64:
-                return launch_flash<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width,
-                                           split_scale, order, s);
+                return launch_flash<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split, order, s);
             default: return CUBERT_UNSUPPORTED;  // head size 128 would spill the accumulators to scratch
         }
     }
     switch (head_size) {
         case 32:
-            return launch_fused<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, split_scale,
+            return launch_fused<T, 32>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split,
                                        s);
         case 64:
-            return launch_fused<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, split_scale,
+            return launch_fused<T, 64>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split,
                                        s);
         default:
-            return launch_fused<T, 128>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split_width, split_scale,
+            return launch_fused<T, 128>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq, split,
                                         s);
     }
 }
@@ -1638,7 +1637,7 @@ extern "C" int cubert_attention_fused_ordered_f32(const float *q, const float *k
                                                   float alpha, int batch, int heads, int seq_length, int head_size,
                                                   void *stream) {
     return cubert::attention_fused<float>(q, k, v, ld, mask, ctx, ld_ctx, alpha, batch, heads, seq_length, head_size,
-                                          stream, 0, 1.f, order);
+                                          stream, cubert::SplitOut(), order);
 }
 
 extern "C" int cubert_attention_fused_ordered_f16(const cubert_half *q, const cubert_half *k, const cubert_half *v, int ld,
@@ -1647,17 +1646,18 @@ extern "C" int cubert_attention_fused_ordered_f16(const cubert_half *q, const cu
                                                   void *stream) {
     return cubert::attention_fused<cubert::half_t>((const cubert::half_t *) q, (const cubert::half_t *) k,
                                                    (const cubert::half_t *) v, ld, mask, (cubert::half_t *) ctx,
-                                                   ld_ctx, alpha, batch, heads, seq_length, head_size, stream, 0, 1.f,
+                                                   ld_ctx, alpha, batch, heads, seq_length, head_size, stream, cubert::SplitOut(),
                                                    order);
 }
 
 extern "C" int cubert_attention_fused_split3_f32(const float *q, const float *k, const float *v, int ld,
                                                 const int8_t *mask, float scale, cubert_half *split_ctx, float alpha,
-                                                int batch, int heads, int seq_length, int head_size, void *stream) {
+                                                int batch, int heads, int seq_length, int head_size, int *overflow,
+                                                void *stream) {
     if (split_ctx != nullptr && !cubert::is_aligned(split_ctx, 2)) return CUBERT_BAD_ARGUMENT;
     const int hidden = heads * head_size;
     return cubert::attention_fused<float>(q, k, v, ld, mask, reinterpret_cast<float *>(split_ctx), hidden, alpha, batch,
-                                          heads, seq_length, head_size, stream, hidden, scale);
+                                          heads, seq_length, head_size, stream, cubert::SplitOut{hidden, scale, overflow});
 }
 
 extern "C" int cubert_attention_fused_f16(const cubert_half *q, const cubert_half *k, const cubert_half *v, int ld,

@@ -47,6 +47,10 @@ __device__ __forceinline__ void split_two_terms(float x, half_t &hi, half_t &lo)
     lo = (half_t) fminf(fmaxf(x - (float) hi, -kMax), kMax);
 }
 
+// Whether split_two_terms had to clamp x (or x is not a number): the two terms then do not add up to x, and whoever
+// consumes them must be told (the kernels that write two-term rows raise a flag the caller looks at).
+__device__ __forceinline__ bool two_term_overflow(float x) { return !(fabsf(x) <= 65504.f); }
+
 // Widest vector (in elements) that is at most 16 bytes.
 template <typename T>
 struct MaxVec {

@@ -49,7 +49,8 @@ __device__ __forceinline__ int uniform_i8(const int8_t *__restrict__ p, int inde
 template <typename T, int VEC, int CHUNKS>
 __device__ __forceinline__ void ln_finish(float (&x)[CHUNKS][VEC], float sum, float sumsq, const Vec<T, VEC> (&g)[CHUNKS],
                                           const Vec<T, VEC> (&b)[CHUNKS], T *__restrict__ out_row, int lane,
-                                          half_t *__restrict__ split_row = nullptr, float split_scale = 1.f) {
+                                          half_t *__restrict__ split_row = nullptr, float split_scale = 1.f,
+                                          int *__restrict__ overflow = nullptr) {
     constexpr int H = kWave * VEC * CHUNKS;
     float mean, rstd;
     ln_stats(sum, sumsq, H, mean, rstd);
@@ -63,10 +64,14 @@ __device__ __forceinline__ void ln_finish(float (&x)[CHUNKS][VEC], float sum, fl
         store_vec<T, VEC>(out_row + (c * kWave + lane) * VEC, o);
         if (split_row != nullptr) {  // (uniform)
             Vec<half_t, VEC> hi, lo;
+            bool over = false;
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
-                split_two_terms(to_f32(o.v[i]) * split_scale, hi.v[i], lo.v[i]);
+                const float y = to_f32(o.v[i]) * split_scale;
+                split_two_terms(y, hi.v[i], lo.v[i]);
+                over = over || two_term_overflow(y);
             }
+            if (over && overflow != nullptr) *overflow = 1;  // the caller recomputes in fp32
             half_t *at = split_row + (c * kWave + lane) * VEC;
             store_vec<half_t, VEC>(at, hi);
             store_vec<half_t, VEC>(at + H, hi);
@@ -79,7 +84,8 @@ template <typename T, int VEC, int CHUNKS, bool HAS_BIAS, bool SPLIT = false>
 __global__ __launch_bounds__(kBlock) void bias_res_ln_kernel(T *__restrict__ inout, const T *__restrict__ residual,
                                                              const T *__restrict__ bias, const T *__restrict__ beta,
                                                              const T *__restrict__ gamma, int rows,
-                                                             half_t *__restrict__ split_out, float split_scale) {
+                                                             half_t *__restrict__ split_out, float split_scale,
+                                                             int *__restrict__ overflow) {
     constexpr int H = kWave * VEC * CHUNKS;
     const int row = blockIdx.x * kRowsPerBlock + wave_in_block();
     if (row >= rows) return;
@@ -118,7 +124,7 @@ __global__ __launch_bounds__(kBlock) void bias_res_ln_kernel(T *__restrict__ ino
         }
     }
     ln_finish<T, VEC, CHUNKS>(x, sum, sumsq, g, be, io, lane, SPLIT ? split_out + (size_t) row * 3 * H : nullptr,
-                              split_scale);
+                              split_scale, overflow);
 }
 
 template <typename T, int VEC, int CHUNKS>
@@ -359,9 +365,9 @@ int bias_res_ln(T *inout, const T *residual, const T *bias, const T *beta, const
     if (hidden == kWave * VEC * CHUNKS && vector_ok<T>(hidden, VEC, {inout, residual, bias, beta, gamma})) { \
         if (bias != nullptr)                                                                             \
             return launch(bias_res_ln_kernel<T, VEC, CHUNKS, true>, grid, block, s, inout, residual, bias, beta, gamma, \
-                          rows, nullptr, 1.f);                                                           \
+                          rows, nullptr, 1.f, nullptr);                                                  \
         return launch(bias_res_ln_kernel<T, VEC, CHUNKS, false>, grid, block, s, inout, residual, bias, beta, gamma, \
-                      rows, nullptr, 1.f);                                                               \
+                      rows, nullptr, 1.f, nullptr);                                                      \
     }
     CUBERT_LN_CASE(V, 1)
     CUBERT_LN_CASE(V, 2)
@@ -382,7 +388,7 @@ int bias_res_ln(T *inout, const T *residual, const T *bias, const T *beta, const
 // bias + residual + LayerNorm of fp32 rows, in place, and the result again as two-term fp16 rows in split_out
 // [rows, 3 * hidden]; only the register-resident shapes (hidden = 256 k), anything else is declined.
 int bias_res_ln_split3(float *inout, const float *residual, const float *bias, const float *beta, const float *gamma,
-                       int rows, int hidden, float scale, half_t *split_out, void *stream) {
+                       int rows, int hidden, float scale, half_t *split_out, int *overflow, void *stream) {
     if (rows < 0 || hidden <= 0 || !inout || !residual || !beta || !gamma || !split_out) return CUBERT_BAD_ARGUMENT;
     if (rows == 0) return 0;
     hipStream_t s = (hipStream_t) stream;
@@ -392,9 +398,9 @@ int bias_res_ln_split3(float *inout, const float *residual, const float *bias, c
     if (hidden == kWave * 4 * CHUNKS && vector_ok<float>(hidden, 4, {inout, residual, bias, beta, gamma})) {         \
         if (bias != nullptr)                                                                                          \
             return launch(bias_res_ln_kernel<float, 4, CHUNKS, true, true>, grid, block, s, inout, residual, bias, beta, \
-                          gamma, rows, split_out, scale);                                                             \
+                          gamma, rows, split_out, scale, overflow);                                                   \
         return launch(bias_res_ln_kernel<float, 4, CHUNKS, false, true>, grid, block, s, inout, residual, bias, beta,  \
-                      gamma, rows, split_out, scale);                                                                 \
+                      gamma, rows, split_out, scale, overflow);                                                       \
     }
     CUBERT_LN_SPLIT_CASE(1)
     CUBERT_LN_SPLIT_CASE(2)
@@ -458,9 +464,9 @@ extern "C" int cubert_bias_res_ln_f32(float *inout, const float *residual, const
 
 extern "C" int cubert_bias_res_ln_split3_f32(float *inout, const float *residual, const float *bias, const float *beta,
                                              const float *gamma, int rows, int hidden, float scale,
-                                             cubert_half *split_out, void *stream) {
+                                             cubert_half *split_out, int *overflow, void *stream) {
     return cubert::bias_res_ln_split3(inout, residual, bias, beta, gamma, rows, hidden, scale,
-                                      (cubert::half_t *) split_out, stream);
+                                      (cubert::half_t *) split_out, overflow, stream);
 }
 
 extern "C" int cubert_bias_res_ln_f16(cubert_half *inout, const cubert_half *residual, const cubert_half *bias,

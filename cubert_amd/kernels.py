@@ -124,7 +124,7 @@ def attention_fused(qkv, mask, batch, heads, seq, head_size, alpha, order=None):
     return ctx
 
 
-def attention_fused_split3(qkv, mask, batch, heads, seq, head_size, alpha, scale=1.0):
+def attention_fused_split3(qkv, mask, batch, heads, seq, head_size, alpha, scale=1.0, overflow=None):
     """attention_fused of an fp32 projection with scale * context as fp16 rows [B*S, 3*H]: hi | hi | lo; None when
     the shape does not fit."""
     hidden = heads * head_size
@@ -132,7 +132,7 @@ def attention_fused_split3(qkv, mask, batch, heads, seq, head_size, alpha, scale
     ctx = torch.empty((batch * seq, 3 * hidden), dtype=torch.float16, device=qkv.device)
     rc = lib().cubert_attention_fused_split3_f32(_ptr(flat), _ptr(flat[hidden:]), _ptr(flat[2 * hidden:]), 3 * hidden,
                                                  _ptr(mask), float(scale), _ptr(ctx), float(alpha), batch, heads, seq, head_size,
-                                                 _stream())
+                                                 _ptr(overflow), _stream())
     if rc == -2:
         return None
     _check(rc, "cubert_attention_fused_split3_f32")
@@ -187,30 +187,32 @@ def classifier_head_(pooled, pooler_bias, weights, out_bias):
     return logits, probs
 
 
-def split3(x, scale=1.0, lo_in_middle=False):
+def split3(x, scale=1.0, lo_in_middle=False, overflow=None):
     """fp32 rows [rows, width] as fp16 rows [rows, 3 * width]: hi | hi | lo (lo_in_middle: hi | lo | hi)."""
     rows, width = x.shape
     out = torch.empty((rows, 3 * width), dtype=torch.float16, device=x.device)
-    _check(lib().cubert_split3_f32(_ptr(x), rows, width, float(scale), int(lo_in_middle), _ptr(out), _stream()),
+    _check(lib().cubert_split3_f32(_ptr(x), rows, width, float(scale), int(lo_in_middle), _ptr(out), _ptr(overflow),
+                                   _stream()),
            "cubert_split3_f32")
     return out
 
 
-def bias_gelu_split3(x, bias, scale=1.0):
+def bias_gelu_split3(x, bias, scale=1.0, overflow=None):
     """scale * GELU(x + bias) of fp32 rows as fp16 rows [rows, 3 * width]: hi | hi | lo."""
     rows, width = x.shape
     out = torch.empty((rows, 3 * width), dtype=torch.float16, device=x.device)
-    _check(lib().cubert_bias_gelu_split3_f32(_ptr(x), _ptr(bias), rows, width, float(scale), _ptr(out), _stream()),
+    _check(lib().cubert_bias_gelu_split3_f32(_ptr(x), _ptr(bias), rows, width, float(scale), _ptr(out),
+                                             _ptr(overflow), _stream()),
            "cubert_bias_gelu_split3_f32")
     return out
 
 
-def bias_res_ln_split3_(inout, residual, bias, beta, gamma, scale=1.0):
+def bias_res_ln_split3_(inout, residual, bias, beta, gamma, scale=1.0, overflow=None):
     """bias_res_ln_ of fp32 rows plus scale * the result as fp16 rows [rows, 3 * hidden]: hi | hi | lo; None when declined."""
     rows, hidden = inout.shape
     out = torch.empty((rows, 3 * hidden), dtype=torch.float16, device=inout.device)
     rc = lib().cubert_bias_res_ln_split3_f32(_ptr(inout), _ptr(residual), _ptr(bias), _ptr(beta), _ptr(gamma), rows,
-                                             hidden, float(scale), _ptr(out), _stream())
+                                             hidden, float(scale), _ptr(out), _ptr(overflow), _stream())
     if rc == -2:
         return None
     _check(rc, "cubert_bias_res_ln_split3_f32")

@@ -256,30 +256,34 @@ int cubert_gemm_f16_f32(void *handle, int transA, int transB, int M, int N, int 
  *   out[r] = [hi(in[r]) | lo(in[r]) | hi(in[r])]      (lo_in_middle = 1: the weight side, rows = output features)
  * each part `width` halves, so that a dot product of a token row with a weight row over 3 * width is
  * hi*hi + hi*lo + lo*hi = the fp32 product up to 2^-22 relative.  Values are clamped to the fp16 range; `scale`
- * (a power of two, undone by the GEMM's alpha) keeps small values out of the fp16 subnormals.
+ * (a power of two, undone by the GEMM's alpha) keeps small values out of the fp16 subnormals.  A value that had
+ * to be clamped (|scale * x| > 65504) or is not a number no longer equals its two terms: this and the three entry
+ * points below then store 1 to *overflow (device memory, or page-locked host memory from cubert_malloc_host;
+ * NULL = not wanted; never written otherwise, so the caller clears it), and the caller must not use the product
+ * (the host classes recompute the request with cubert_gemm_f32).
  * replaces: nothing in the reference by itself; it is the operand preparation of the opt-in form of
  * Dense<float>::compute (reference src/cuBERT/op/Dense.cpp:47-57) that runs on the fp16 matrix cores. */
 int cubert_split3_f32(const float *in, int rows, int width, float scale, int lo_in_middle, cubert_half *out,
-                      void *stream);
+                      int *overflow, void *stream);
 /* bias + GELU as cubert_bias_gelu_f32 computes it, times `scale` (a power of two), written as [hi | hi | lo] rows
  * for the GEMM that follows instead of in place.  replaces: gelu<float>, reference src/cuBERT/op/GELU.h:6-7 (op/GELU.cu:14-26), followed
  * by the operand preparation above. */
 int cubert_bias_gelu_split3_f32(const float *in, const float *bias, int rows, int width, float scale,
-                                cubert_half *out, void *stream);
+                                cubert_half *out, int *overflow, void *stream);
 /* cubert_attention_fused_f32 with the context, times `scale` (a power of two), written as [hi | hi | lo] rows,
  * split_ctx[batch * seq_length, 3 * heads * head_size], for the GEMM that follows, instead of as fp32.  Same shape limits and return codes.
  * replaces: AttentionSelf<float>::_in_compute between the projections, reference
  * src/cuBERT/op_att/AttentionSelf.cpp:96-111, followed by the operand preparation above. */
 int cubert_attention_fused_split3_f32(const float *q, const float *k, const float *v, int ld, const int8_t *mask,
                                       float scale, cubert_half *split_ctx, float alpha, int batch, int heads, int seq_length,
-                                      int head_size, void *stream);
+                                      int head_size, int *overflow, void *stream);
 /* cubert_bias_res_ln_f32, and its result times `scale` (a power of two) again as [hi | hi | lo] rows in
  * split_out[rows, 3 * hidden] for the GEMM that follows.  hidden must be 256 k (k = 1..6, 8) with 16-byte aligned operands, otherwise CUBERT_UNSUPPORTED is
  * returned and nothing is done.  replaces: layer_norm_<float>, reference src/cuBERT/op/LayerNorm.h:5-14
  * (op/LayerNorm.cu:11-100), followed by the operand preparation above. */
 int cubert_bias_res_ln_split3_f32(float *inout, const float *residual, const float *bias, const float *beta,
                                   const float *gamma, int rows, int hidden, float scale, cubert_half *split_out,
-                                  void *stream);
+                                  int *overflow, void *stream);
 
 /* C = alpha * A * B + bias for N <= 32 columns (no transposes, beta = 0): the Dense layer of a request with at
  * most 32 tokens, where A is the [in, out] weight matrix (M = out, K = in) and each column of B one token.

@@ -503,6 +503,66 @@ def test_attention_fused_split3_equals_attention_then_split(K, batch, heads, seq
     assert torch.equal(got, K.split3(plain, 16.0))  # the same context values, written in the other form
 
 
+def test_two_term_kernels_raise_the_overflow_flag(K):
+    """A value whose scaled form is beyond the fp16 range (or is not a number) cannot be written as two fp16 terms:
+    each of the four kernels that write two-term rows stores 1 to the caller's flag then, and leaves it alone
+    otherwise (the host classes recompute such a request with the fp32 GEMMs)."""
+    rng = np.random.default_rng(5)
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+    def raised():
+        torch.cuda.synchronize()
+        v = int(flag.item())
+        flag.zero_()
+        return v
+
+    # plain rows: vector path (width 768) and element path (width 7)
+    for width in (768, 7):
+        x = rng.normal(0, 1, (9, width)).astype(np.float32)
+        K.split3(dev(x), 16.0, overflow=flag)
+        assert raised() == 0
+        x[4, width - 2] = 4094.1                      # 16 x = 65505.6 > 65504
+        K.split3(dev(x), 16.0, overflow=flag)
+        assert raised() == 1
+        x[4, width - 2] = -4093.9                     # 16 x = -65502.4: still representable
+        K.split3(dev(x), 16.0, overflow=flag)
+        assert raised() == 0
+        x[0, 0] = np.nan
+        K.split3(dev(x), 16.0, overflow=flag)
+        assert raised() == 1
+        K.split3(dev(x), 16.0)                        # no flag wanted: nothing to write to
+    # bias + GELU
+    x = rng.normal(0, 1, (5, 768)).astype(np.float32)
+    b = rng.normal(0, 1, 768).astype(np.float32)
+    K.bias_gelu_split3(dev(x), dev(b), 16.0, overflow=flag)
+    assert raised() == 0
+    x[2, 100] = 5000.0                                # GELU(5000 + b) = 5000 + b
+    K.bias_gelu_split3(dev(x), dev(b), 16.0, overflow=flag)
+    assert raised() == 1
+    x[2, 100] = -5000.0                               # GELU of a large negative number is 0
+    K.bias_gelu_split3(dev(x), dev(b), 16.0, overflow=flag)
+    assert raised() == 0
+    # bias + residual + LayerNorm: outputs are gamma * (unit variance) + beta
+    x = rng.normal(0, 1, (6, 768)).astype(np.float32)
+    res = rng.normal(0, 1, (6, 768)).astype(np.float32)
+    gamma, beta = np.ones(768, np.float32), np.zeros(768, np.float32)
+    assert K.bias_res_ln_split3_(dev(x), dev(res), None, dev(beta), dev(gamma), 16.0, overflow=flag) is not None
+    assert raised() == 0
+    gamma[17] = 30000.0
+    assert K.bias_res_ln_split3_(dev(x), dev(res), None, dev(beta), dev(gamma), 16.0, overflow=flag) is not None
+    assert raised() == 1
+    # attention: the context is an average of V rows, so a large V column carries through
+    batch, heads, seq, d = 3, 4, 32, 64
+    hidden = heads * d
+    qkv = rng.normal(0, 1, (batch * seq, 3 * hidden)).astype(np.float32)
+    mask = torch.ones((batch, seq), dtype=torch.int8, device="cuda")
+    assert K.attention_fused_split3(dev(qkv), mask, batch, heads, seq, d, 0.125, scale=16.0, overflow=flag) is not None
+    assert raised() == 0
+    qkv[:, 2 * hidden + 5] = 6000.0
+    assert K.attention_fused_split3(dev(qkv), mask, batch, heads, seq, d, 0.125, scale=16.0, overflow=flag) is not None
+    assert raised() == 1
+
+
 def test_bias_res_ln_split3_declines_other_hidden_sizes(K):
     x = dev(np.zeros((2, 100), np.float32))
     v = dev(np.ones(100, np.float32))
@@ -877,15 +937,15 @@ def test_empty_and_bad_arguments(K):
     assert L.cubert_mean_pool_f32(x.data_ptr(), x.data_ptr(), 1, 0, 768, None) == -1
     # the two-term operand kernels
     h = torch.zeros((4, 3 * 768), dtype=torch.float16, device="cuda")
-    assert L.cubert_split3_f32(x.data_ptr(), 0, 768, 1.0, 0, h.data_ptr(), None) == 0
-    assert L.cubert_split3_f32(x.data_ptr(), 4, 0, 1.0, 0, h.data_ptr(), None) == -1
-    assert L.cubert_split3_f32(None, 4, 768, 1.0, 0, h.data_ptr(), None) == -1
-    assert L.cubert_bias_gelu_split3_f32(x.data_ptr(), None, 0, 768, 1.0, h.data_ptr(), None) == 0
-    assert L.cubert_bias_gelu_split3_f32(x.data_ptr(), None, 4, 768, 1.0, None, None) == -1
+    assert L.cubert_split3_f32(x.data_ptr(), 0, 768, 1.0, 0, h.data_ptr(), None, None) == 0
+    assert L.cubert_split3_f32(x.data_ptr(), 4, 0, 1.0, 0, h.data_ptr(), None, None) == -1
+    assert L.cubert_split3_f32(None, 4, 768, 1.0, 0, h.data_ptr(), None, None) == -1
+    assert L.cubert_bias_gelu_split3_f32(x.data_ptr(), None, 0, 768, 1.0, h.data_ptr(), None, None) == 0
+    assert L.cubert_bias_gelu_split3_f32(x.data_ptr(), None, 4, 768, 1.0, None, None, None) == -1
     assert L.cubert_bias_res_ln_split3_f32(x.data_ptr(), x.data_ptr(), None, x.data_ptr(), x.data_ptr(), 0, 768, 1.0,
-                                           h.data_ptr(), None) == 0
+                                           h.data_ptr(), None, None) == 0
     assert L.cubert_bias_res_ln_split3_f32(x.data_ptr(), x.data_ptr(), None, x.data_ptr(), x.data_ptr(), 4, 768, 1.0,
-                                           None, None) == -1
+                                           None, None, None) == -1
     torch.cuda.synchronize()
 
 

@@ -166,9 +166,12 @@ CONFIG_CASES = [
 ]
 
 
+@pytest.mark.parametrize("two_term", [False, True])
 @pytest.mark.parametrize("seed", [11, 12, 13])
-def test_randomly_drawn_model_configurations(cb, seed):
-    """Fifteen models per seed with every size drawn at random -- heads, head size (also ones no matrix-core kernel
+def test_randomly_drawn_model_configurations(cb, seed, two_term, monkeypatch):
+    """(two_term: the same draws with CUBERT_FP32_DENSE=f16x3 in the environment, fp32 cases only -- requests of at
+    least 384 tokens then run their Dense layers on the fp16 matrix cores from two-term operands, same bound.)
+    Fifteen models per seed with every size drawn at random -- heads, head size (also ones no matrix-core kernel
     takes), seq_length (1 ... 512, not only multiples of 32), intermediate size, layers, labels (few and many), with and
     without pooler / classifier / classifier bias, both compute types, prefix and scattered masks, a batch below the
     maximum -- against the oracle, every output; two calls in a row must agree bit for bit.  The fp32 bound here is
@@ -176,6 +179,8 @@ def test_randomly_drawn_model_configurations(cb, seed):
     oracle itself is up to 1e-5 away from a float64 evaluation (summation order over 1536 ... 3080 terms), so two fp32
     evaluations are up to 3e-5 apart (measured over 480 drawn models: 2.8e-5; fp16: 1.3e-2)."""
     from cubert_amd.testing import random_bert_weights, random_inputs
+    if two_term:
+        monkeypatch.setenv("CUBERT_FP32_DENSE", "f16x3")
     rng = np.random.default_rng(seed)
     for case in range(15):
         heads = int(rng.choice([1, 2, 3, 4, 8, 12]))
@@ -196,6 +201,8 @@ def test_randomly_drawn_model_configurations(cb, seed):
         what = "seed %d case %d: B=%d/%d S=%d H=%d A=%d I=%d L=%d labels=%d pooler=%s classifier=%s bias=%s %s %s" % (
             seed, case, batch, max_batch, seq, hidden, heads, inter, layers, labels, pooler, classifier, cbias,
             "f16" if compute_type else "f32", "scattered" if scattered else "prefix")
+        if two_term and compute_type == 1:
+            continue
         print(what, flush=True)
         w = random_bert_weights(seed=seed * 100 + case, vocab=vocab, hidden=hidden, layers=layers, heads=heads,
                                 intermediate=inter, max_position=max(seq, 8), type_vocab=2, labels=labels, pooler=pooler,
@@ -483,6 +490,45 @@ def test_models_per_gpu_must_be_a_sane_count(cb, small_pb, monkeypatch):
         monkeypatch.setenv("CUBERT_MODELS_PER_GPU", bad)
         with pytest.raises(ValueError):
             cb.Model(path, 4, 32, 3, 4)
+
+
+def test_two_term_dense_falls_back_to_fp32_when_an_activation_does_not_fit(cb, monkeypatch):
+    """CUBERT_FP32_DENSE=f16x3 with a model whose LayerNorm scales push activations beyond what two fp16 terms can
+    hold (|16 x| > 65504): the request is recomputed on the fp32 GEMMs and its outputs are, bit for bit, those of the
+    same model opened without the variable; a request that fits still runs (and stays within 1e-5 of the oracle) in the
+    two-term form afterwards."""
+    from cubert_amd.testing import random_bert_weights, random_inputs
+    w = random_bert_weights(seed=23, labels=3, pooler=True, classifier=True, classifier_bias=True, ln_random=True,
+                            **SMALL)
+    big = dict(w)
+    name = "bert/encoder/layer_1/attention/output/LayerNorm/gamma"
+    big[name] = (w[name] * 9000.0).astype(np.float32)            # that layer's LayerNorm outputs reach ~ 3e4
+    ids, mask, seg = random_inputs(seed=24, batch=13, seq_length=32, vocab=SMALL["vocab"], min_valid=2,
+                                   segment_split="random", scattered_mask=True)
+    plain = cb.Bert(big, 14, 32, 3, 4)
+    want_big = plain.forward(ids, mask, seg)
+    plain.close()
+    monkeypatch.setenv("CUBERT_FP32_DENSE", "f16x3")
+    for weights, expect_fallback in ((big, True), (w, False)):
+        bert = cb.Bert(weights, 14, 32, 3, 4)
+        bert.profile(["dense_split", "dense_gemm"])
+        got = bert.forward(ids, mask, seg)                       # 416 tokens: the two-term form applies
+        counts = bert.profile_read()
+        assert counts["dense_split"][1] >= 1                     # ... and was tried
+        if expect_fallback:
+            # tried (4 GEMMs per layer + pooler and classifier), then all of it again in fp32
+            assert counts["dense_gemm"][1] >= 2 * 4 * 3, counts
+            for k in ("embedding_output", "sequence_output", "pooled_output", "logits", "probs"):
+                assert np.array_equal(got[k].view(np.uint32), want_big[k].view(np.uint32)), k
+            # single outputs through the other output methods take the same route
+            again = bert.forward(ids, mask, seg)
+            assert np.array_equal(again["logits"].view(np.uint32), want_big["logits"].view(np.uint32))
+        else:
+            assert counts["dense_gemm"][1] < 2 * 4 * 3, counts
+            want = oracle.bert_forward(weights, ids, mask, seg, 3, 4)
+            for k in ("embedding_output", "sequence_output", "pooled_output", "logits", "probs"):
+                assert_close(got[k], want[k], FP32_TOL, "two-term " + k)
+        bert.close()
 
 
 def test_first_request_does_not_pay_for_gemm_planning(cb):
