@@ -189,7 +189,7 @@ void Transformer<T>::layout_buffers() {
     qkv_ld = 3 * H + 64;
     qkv_out = buffers.take<T>(M * qkv_ld);
     context_out = buffers.take<T>(M * H);
-    attention_order = buffers.take<int>(max_batch_size);
+    attention_order = buffers.take<int>(8 * max_batch_size);  // indices, then a record of live tiles per position
     attention_output = buffers.take<T>(M * H);
     intermediate_output = buffers.take<T>(M * intermediate_size);
     layer_output[0] = buffers.take<T>(M * H);

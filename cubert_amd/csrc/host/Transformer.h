@@ -133,7 +133,7 @@ private:
     T *qkv_out;              // [M, qkv_ld]
     T *attention_scores = nullptr;  // [B, heads, seq, seq], in score_memory (null until scores() is first called)
     T *context_out;          // [M, hidden]
-    int *attention_order = nullptr;  // [max_batch]: sequence indices, most live key tiles first (seq_length > 128)
+    int *attention_order = nullptr;  // [8 * max_batch]: sequence indices, most live key tiles first, and their tile lists (seq_length > 128)
     bool order_ready = false;        // attention_order holds the current request's order
     T *attention_output;     // [M, hidden]
     T *intermediate_output;  // [M, intermediate]

@@ -1076,7 +1076,7 @@ template <typename T, int D, bool SPLIT>
 __global__ __launch_bounds__(1024) void attention_flash_grouped_kernel(
     const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, int ld, const int8_t *__restrict__ mask,
     T *__restrict__ ctx, int ld_ctx, float alpha, int heads, int skip_masked_tiles, SplitOut split,
-    const int *__restrict__ order) {
+    const int *__restrict__ order, int order_has_records) {
     constexpr int V = Mma<T>::kVec;
     constexpr int kSteps = D / 2 / V;
     constexpr int kColTiles = D / 32;
@@ -1111,19 +1111,35 @@ __global__ __launch_bounds__(1024) void attention_flash_grouped_kernel(
 #pragma unroll
     for (int t = 0; t < kSteps; ++t) qv[t] = load_vec<T, V>(q_row + t * V);
 
-    // bit kt: key tile kt has an unmasked key (workgroup-uniform: scalar loads of the mask row as words)
-    unsigned live = 0;
-    if (mask != nullptr && skip_masked_tiles) {
-        const uint32_t *words = reinterpret_cast<const uint32_t *>(mask + (size_t) b * S);
-        for (int kt = 0; kt < KT; ++kt) {
-            uint32_t any = 0;
+    // The live key tiles (those with an unmasked key) as a list: n_live tile numbers in ascending order, 4 bits each.
+    // With an order array that carries records (attention_order writes them) the list of this sequence is one scalar
+    // load next to the one for `b`; otherwise it is made here from the mask row, read as words with scalar loads
+    // (workgroup-uniform either way).
+    int n_live = 0;
+    unsigned long long tile_list = 0;
+    if (order != nullptr && order_has_records && mask != nullptr && skip_masked_tiles) {
+        const int batch = (int) gridDim.x / heads;
+        const int *rec = order + 4 * (size_t) batch + 4 * (size_t) rank;
+        n_live = rec[0];
+        tile_list = (unsigned long long) (unsigned) rec[1] | ((unsigned long long) (unsigned) rec[2] << 32);
+    } else {
+        if (mask != nullptr && skip_masked_tiles) {
+            const uint32_t *words = reinterpret_cast<const uint32_t *>(mask + (size_t) b * S);
+            for (int kt = 0; kt < KT; ++kt) {
+                uint32_t any = 0;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) any |= words[kt * 8 + i];
-            live |= (any != 0 ? 1u : 0u) << kt;
+                for (int i = 0; i < 8; ++i) any |= words[kt * 8 + i];
+                if (any != 0) tile_list |= (unsigned long long) kt << (4 * n_live++);
+            }
+        }
+        if (n_live == 0) {  // no mask, or no kept key at all: every tile
+            n_live = KT;
+            tile_list = 0xfedcba9876543210ull;
         }
     }
-    if (live == 0) live = KT >= 32 ? ~0u : (1u << KT) - 1u;
-    live = __builtin_amdgcn_readfirstlane(live);
+    n_live = __builtin_amdgcn_readfirstlane(n_live);
+    tile_list = (unsigned long long) (unsigned) __builtin_amdgcn_readfirstlane((int) (unsigned) tile_list) |
+                ((unsigned long long) (unsigned) __builtin_amdgcn_readfirstlane((int) (unsigned) (tile_list >> 32)) << 32);
 
     for (int i = threadIdx.x; i < S; i += kThreads) {
         s_mask[i] = (mask != nullptr && !mask[(size_t) b * S + i]) ? kMaskedScore * kLog2e : 0.f;
@@ -1137,21 +1153,11 @@ __global__ __launch_bounds__(1024) void attention_flash_grouped_kernel(
     for (int jt = 0; jt < kColTiles; ++jt) out[jt] = v16f32{};
     bool first_chunk = true;
 
-    for (unsigned todo = live; todo != 0;) {
+    for (int g0 = 0; g0 < n_live; g0 += G) {
         // the next group: the lowest G live tiles that are left
-        unsigned group = 0;
-        for (int i = 0; i < G && todo != 0; ++i) {
-            const unsigned low = todo & (0u - todo);
-            group |= low;
-            todo ^= low;
-        }
-        const int in_group = __builtin_popcount(group);
-        // tile of slot s: the s-th set bit of group (wavefront-uniform: a wavefront's 64 vectors lie in one tile)
-        auto tile_of = [&](int slot) {
-            unsigned rest = group;
-            for (int i = 0; i < slot; ++i) rest &= rest - 1;
-            return __builtin_ctz(rest);
-        };
+        const int in_group = n_live - g0 < G ? n_live - g0 : G;
+        // tile of slot s of this group (wavefront-uniform: a wavefront's 64 vectors lie in one tile)
+        auto tile_of = [&](int slot) { return (int) ((tile_list >> (4 * (g0 + slot))) & 15u); };
         Vec<T, V> kreg[kLoads], vreg[kLoads];
 #pragma unroll
         for (int u = 0; u < kLoads; ++u) {
@@ -1190,18 +1196,13 @@ __global__ __launch_bounds__(1024) void attention_flash_grouped_kernel(
             store_vec<T, V>(s_vt + j * kPitchV + grp * V, vreg[u]);
         }
         __syncthreads();
-        int slot0 = 0;
-        for (unsigned rest = group; rest != 0;) {  // the group's tiles in ascending order, kChunk per step
+        for (int s0 = 0; s0 < in_group; s0 += kChunk) {  // the group's tiles in ascending order, kChunk per step
             int tiles[kChunk], slots[kChunk];
 #pragma unroll
             for (int cc = 0; cc < kChunk; ++cc) {
-                tiles[cc] = -1;
-                slots[cc] = 0;
-                if (rest != 0) {
-                    tiles[cc] = __builtin_ctz(rest);
-                    slots[cc] = slot0++;
-                    rest &= rest - 1;
-                }
+                const bool present = s0 + cc < in_group;
+                tiles[cc] = present ? tile_of(s0 + cc) : -1;
+                slots[cc] = present ? s0 + cc : 0;
             }
             v16f32 p[kChunk];
             float cm = -3.402823466e+38f;
@@ -1306,9 +1307,14 @@ __global__ __launch_bounds__(1024) void attention_flash_grouped_kernel(
 // kernels then take sequence order[blockIdx / heads].  Results do not depend on the order in any way.
 constexpr int kOrderMaxBatch = 4096;
 
+// order[0 .. batch): the sequence indices, most live tiles first.  order[4 * batch + 4 * i ...]: a record for the
+// sequence at position i -- {number of live tiles, their tile numbers in ascending order 4 bits each (low word, high
+// word), the live tiles as a bit mask} -- so that a long-sequence kernel gets its list of tiles with one scalar load
+// instead of reading the mask row again.  8 * batch ints in all.
 __global__ __launch_bounds__(kBlock) void attention_order_kernel(const int8_t *__restrict__ mask, int batch, int seq,
                                                                  int *__restrict__ order) {
     __shared__ unsigned char tiles_of[kOrderMaxBatch];
+    __shared__ unsigned short bits_of[kOrderMaxBatch];
     __shared__ int bucket[20];  // [t]: sequences with t live tiles (t <= 16), then their first position
     const int key_tiles = seq / 32;
     if (threadIdx.x < 20) bucket[threadIdx.x] = 0;
@@ -1316,14 +1322,20 @@ __global__ __launch_bounds__(kBlock) void attention_order_kernel(const int8_t *_
     for (int b = threadIdx.x; b < batch; b += kBlock) {
         const uint32_t *words = reinterpret_cast<const uint32_t *>(mask + (size_t) b * seq);
         int live = 0;
+        unsigned bits = 0;
         for (int kt = 0; kt < key_tiles; ++kt) {
             uint32_t any = 0;
 #pragma unroll
             for (int i = 0; i < 8; ++i) any |= words[kt * 8 + i];
             live += any != 0;
+            bits |= (any != 0 ? 1u : 0u) << kt;
         }
-        if (live == 0) live = key_tiles;  // no kept key: the kernels compute every tile
+        if (live == 0) {  // no kept key: the kernels compute every tile
+            live = key_tiles;
+            bits = (1u << key_tiles) - 1u;
+        }
         tiles_of[b] = (unsigned char) live;
+        bits_of[b] = (unsigned short) bits;
         atomicAdd(&bucket[live], 1);
     }
     __syncthreads();
@@ -1336,13 +1348,29 @@ __global__ __launch_bounds__(kBlock) void attention_order_kernel(const int8_t *_
         }
     }
     __syncthreads();
-    for (int b = threadIdx.x; b < batch; b += kBlock) order[atomicAdd(&bucket[tiles_of[b]], 1)] = b;
+    for (int b = threadIdx.x; b < batch; b += kBlock) {
+        const int at = atomicAdd(&bucket[tiles_of[b]], 1);
+        order[at] = b;
+        const unsigned bits = bits_of[b];
+        unsigned long long list = 0;
+        int n = 0;
+        for (int kt = 0; kt < key_tiles; ++kt) {
+            if ((bits >> kt) & 1u) list |= (unsigned long long) kt << (4 * n++);
+        }
+        int *rec = order + 4 * (size_t) batch + 4 * (size_t) at;
+        rec[0] = n;
+        rec[1] = (int) (unsigned) list;
+        rec[2] = (int) (unsigned) (list >> 32);
+        rec[3] = (int) bits;
+    }
 }
 
 int attention_order(const int8_t *mask, int batch, int seq, int *order, void *stream) {
     if (!mask || !order || batch < 0 || seq <= 0) return CUBERT_BAD_ARGUMENT;
     if (batch == 0) return 0;
-    if (seq % 32 != 0 || seq > 512 || batch > kOrderMaxBatch || !is_aligned(mask, 4)) return CUBERT_UNSUPPORTED;
+    if (seq % 32 != 0 || seq > 512 || batch > kOrderMaxBatch || !is_aligned(mask, 4) || !is_aligned(order, 16)) {
+        return CUBERT_UNSUPPORTED;
+    }
     return launch_untimed(attention_order_kernel, dim3(1), dim3(kBlock), 0u, (hipStream_t) stream, mask, batch, seq,
                           order);
 }
@@ -1531,19 +1559,25 @@ int launch_flash(const T *q, const T *k, const T *v, int ld, const int8_t *mask,
     static const bool whole_head = getenv("CUBERT_FLASH_WHOLE") != nullptr;
     if (seq == 512 && !whole_head) {
         constexpr int G = 32 * V / D;
+        // CUBERT_FLASH_RECORDS=0 in the environment: the kernel reads the mask row itself instead of the order array's
+        // records (for comparison)
+        static const int use_records = [] {
+            const char *e = std::getenv("CUBERT_FLASH_RECORDS");
+            return e != nullptr && std::string(e) == "0" ? 0 : 1;
+        }();
         const size_t grouped_lds = ((size_t) G * 32 * (D + V) + (size_t) D * (G * 32 + V)) * sizeof(T) +
                                    ((size_t) seq + 16 * 32) * sizeof(float);
         if constexpr (sizeof(T) == 4) {
             if (split.width > 0) {
                 return launch_lds(attention_flash_grouped_kernel<T, D, true>, dim3(batch * heads), dim3(1024),
                                       (unsigned) grouped_lds, s, q, k, v, ld, mask, ctx, ld_ctx, alpha, heads,
-                                      skip_masked_tiles, split, order);
+                                      skip_masked_tiles, split, order, use_records);
             }
         }
         if (split.width > 0) return CUBERT_UNSUPPORTED;
         return launch_lds(attention_flash_grouped_kernel<T, D, false>, dim3(batch * heads), dim3(1024),
                               (unsigned) grouped_lds, s, q, k, v, ld, mask, ctx, ld_ctx, alpha, heads, skip_masked_tiles,
-                              split, order);
+                              split, order, use_records);
     }
     if (lds > 160 * 1024) return CUBERT_UNSUPPORTED;
     if constexpr (sizeof(T) == 4) {

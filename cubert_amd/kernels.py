@@ -90,10 +90,11 @@ def attention_scores(qkv, batch, heads, seq, head_size, alpha):
 
 
 def attention_order(mask):
-    """Sequence indices by falling number of key tiles (32 keys) with a kept key, as an int32 tensor; None when the
-    shape or the mask's alignment is not taken."""
+    """What cubert_attention_order writes, as an int32 tensor of 8 * batch: the sequence indices by falling number of
+    key tiles (32 keys) with a kept key in [0, batch), and from 4 * batch on a record of 4 ints per position (live
+    tiles: count, list, bit mask); None when the shape or the mask's alignment is not taken."""
     batch, seq = mask.shape
-    order = torch.empty(batch, dtype=torch.int32, device=mask.device)
+    order = torch.zeros(8 * batch, dtype=torch.int32, device=mask.device)
     rc = lib().cubert_attention_order(_ptr(mask), batch, seq, _ptr(order), _stream())
     if rc == -2:
         return None

@@ -129,12 +129,16 @@ int cubert_attention_fused_f16(const cubert_half *q, const cubert_half *k, const
 /* Longest sequences first.  The long-sequence kernels (seq_length > 128) leave out key tiles (32 keys) whose mask
  * bytes are all zero, so a workgroup's time goes with its sequence's number of live tiles, and workgroups are handed
  * to the compute units in index order: a long sequence late in the batch starts late and the launch waits for it.
- * cubert_attention_order writes the sequence indices 0..batch-1 by falling live-tile count into order[batch] (one
- * small launch; the mask is the same for every layer of a forward pass, so once per pass);
- * cubert_attention_fused_ordered_* is cubert_attention_fused_* taking sequence order[i] where it would take i
- * (order may be NULL: batch order; shapes of at most 128 keys ignore it).  Results are identical with any order.
+ * cubert_attention_order writes the sequence indices 0..batch-1 by falling live-tile count into order[0 .. batch) and,
+ * from order[4 * batch] on, a record of 4 ints for the sequence at each position {number of live tiles, their tile
+ * numbers in ascending order 4 bits each (low word, high word), the live tiles as a bit mask}: `order` holds
+ * 8 * batch ints and is 16-byte aligned (one small launch; the mask is the same for every layer of a forward pass,
+ * so once per pass).  cubert_attention_fused_ordered_* is cubert_attention_fused_* taking sequence order[i] where it
+ * would take i, and the tiles to compute from that position's record (order may be NULL: batch order, tiles from
+ * the mask; shapes of at most 128 keys ignore it).  Results are identical with any order, i.e. with any permutation
+ * of the positions that moves the records along with the indices.
  * CUBERT_UNSUPPORTED from cubert_attention_order (seq_length not a multiple of 32 or above 512, more than 4096
- * sequences, a mask that is not 4-byte aligned): pass NULL.
+ * sequences, a mask that is not 4-byte aligned, an order array that is not 16-byte aligned): pass NULL.
  * No counterpart in the reference, which computes every key of every sequence (src/cuBERT/op_att/AttentionSelf.cpp:96-111). */
 int cubert_attention_order(const int8_t *mask, int batch, int seq_length, int *order, void *stream);
 int cubert_attention_fused_ordered_f32(const float *q, const float *k, const float *v, int ld, const int8_t *mask,

@@ -798,17 +798,28 @@ def test_attention_longest_sequences_first(K, name, batch, heads, seq, d):
     mask[3, ::37] = 1                                  # kept keys scattered over every tile
     dmask = dev(mask)
     order = K.attention_order(dmask)
-    assert order is not None
-    got = order.cpu().numpy().astype(np.int64)
+    assert order is not None and order.numel() == 8 * batch
+    host_order = order.cpu().numpy().astype(np.int64)
+    got = host_order[:batch]
     assert sorted(got.tolist()) == list(range(batch))
-    live = (mask.reshape(batch, seq // 32, 32) != 0).any(-1).sum(-1)
-    live[live == 0] = seq // 32
+    tile_live = (mask.reshape(batch, seq // 32, 32) != 0).any(-1)
+    tile_live[~tile_live.any(-1)] = True               # no kept key at all: every tile
+    live = tile_live.sum(-1)
     assert (np.diff(live[got]) <= 0).all(), live[got]
+    # the record of each position: number of live tiles, their numbers 4 bits each, and as a bit mask
+    records = host_order[4 * batch:].reshape(batch, 4)
+    for position, b in enumerate(got):
+        tiles = np.flatnonzero(tile_live[b])
+        n, lo, hi, bits = (int(v) & 0xffffffff for v in records[position])
+        listed = [((lo | (hi << 32)) >> (4 * i)) & 15 for i in range(n)]
+        assert n == len(tiles) and listed == tiles.tolist() and bits == sum(1 << int(t) for t in tiles), (position, b)
     qkv = dev(q(rng.normal(0, 1, (batch * seq, 3 * H)), name), tdt(name))
     alpha = 1.0 / math.sqrt(d)
     plain = K.attention_fused(qkv, dmask, batch, heads, seq, d, alpha)
     ordered = K.attention_fused(qkv, dmask, batch, heads, seq, d, alpha, order=order)
-    backwards = K.attention_fused(qkv, dmask, batch, heads, seq, d, alpha, order=order.flip(0).contiguous())
+    # any permutation of the positions that moves the records along with the indices
+    flipped = torch.cat([order[:batch].flip(0), order[batch:4 * batch], order[4 * batch:].reshape(batch, 4).flip(0).reshape(-1)])
+    backwards = K.attention_fused(qkv, dmask, batch, heads, seq, d, alpha, order=flipped.contiguous())
     assert plain is not None and ordered is not None and backwards is not None
     assert torch.equal(plain, ordered) and torch.equal(plain, backwards)
     # shapes and masks the sort declines
