@@ -51,46 +51,46 @@ TRAFFIC_PROFILE = "profiles/traffic_pmc.md"
 TRAFFIC_SOURCE = {  # kernel kind -> (source file under cubert_amd/csrc/kernels, first 16 hex digits of its SHA-256)
     "bias_gelu": ("elementwise.hip", "59dcc33f61344079"),
     "bias_tanh": ("elementwise.hip", "59dcc33f61344079"),
-    "bias_res_ln": ("layernorm.hip", "4c00fd91a55914b9"),
-    "embed_ln": ("layernorm.hip", "4c00fd91a55914b9"),
+    "bias_res_ln": ("layernorm.hip", "0adeeda2d66610ed"),
+    "embed_ln": ("layernorm.hip", "0adeeda2d66610ed"),
     "mask_scale_softmax": ("softmax.hip", "90a529eac55169fa"),
     "mean_pool": ("elementwise.hip", "59dcc33f61344079"),
     "classifier_head": ("elementwise.hip", "59dcc33f61344079"),
-    "attention_fused": ("attention.hip", "fd800e8d4c9ccee9"),
+    "attention_fused": ("attention.hip", "f321b185290e9be1"),
 }
 MEASURED_TRAFFIC = {
     "C1": {
-        "embed_ln": 25318195,
-        "attention_fused": 50098109,
-        "bias_res_ln": 37618237,
-        "bias_gelu": 100340642,
-        "classifier_head": 934243,
-        "mask_scale_softmax": 12589795
+        "embed_ln": 25327943,
+        "attention_fused": 50081939,
+        "bias_res_ln": 37631180,
+        "bias_gelu": 100340690,
+        "classifier_head": 934418,
+        "mask_scale_softmax": 12589830
     },
     "C2": {
-        "embed_ln": 12906209,
-        "attention_fused": 25138580,
-        "bias_res_ln": 18866004,
-        "bias_gelu": 50185062,
-        "mean_pool": 6324895,
-        "classifier_head": 147215,
-        "mask_scale_softmax": 25117455
+        "embed_ln": 12910688,
+        "attention_fused": 25138615,
+        "bias_res_ln": 18866015,
+        "bias_gelu": 50185069,
+        "mean_pool": 6325072,
+        "classifier_head": 147249,
+        "mask_scale_softmax": 25117442
     },
     "C3": {
-        "embed_ln": 99789147,
-        "attention_fused": 130327065,
-        "bias_res_ln": 150209246,
-        "bias_gelu": 400910315,
-        "classifier_head": 308663,
-        "mask_scale_softmax": 801925601
+        "embed_ln": 99752919,
+        "attention_fused": 128669232,
+        "bias_res_ln": 150207822,
+        "bias_gelu": 400908701,
+        "classifier_head": 308800,
+        "mask_scale_softmax": 801925779
     },
     "C4": {
-        "embed_ln": 133804718,
-        "attention_fused": 267259400,
-        "bias_res_ln": 200205923,
-        "bias_gelu": 534518836,
-        "classifier_head": 1199487,
-        "mask_scale_softmax": 267503616
+        "embed_ln": 133771994,
+        "attention_fused": 267267591,
+        "bias_res_ln": 200189715,
+        "bias_gelu": 534518904,
+        "classifier_head": 1199624,
+        "mask_scale_softmax": 267503655
     }
 }
 
