@@ -119,7 +119,11 @@ def test_calls_leave_free_device_memory_unchanged(L, context):
     def call(m, n, k):
         return L.cubert_gemm_skinny_noalloc_f32(stream, m, n, k, 1.0, d.ptrs[0], m, d.ptrs[1], k, d.ptrs[2], m, None, 0)
 
-    assert call(M, N, K) == 0                       # first call: set-up done
+    # every kind of call once first: the first call on the device looks up the array's address, and a kernel variant's
+    # first launch is the runtime's business, not this entry point's
+    assert call(M, N, K) == 0
+    assert call(96, 5, 256) == 0
+    assert call(32, 33, 16) == UNSUPPORTED
     assert L.cubert_stream_synchronize(stream) == 0
     before = free_device_bytes(L)
     for _ in range(20):
