@@ -1122,6 +1122,10 @@ __global__ __launch_bounds__(1024) void attention_flash_grouped_kernel(
         const int *rec = order + 4 * (size_t) batch + 4 * (size_t) rank;
         n_live = rec[0];
         tile_list = (unsigned long long) (unsigned) rec[1] | ((unsigned long long) (unsigned) rec[2] << 32);
+        if (n_live < 1 || n_live > KT) {  // not a record attention_order wrote: every tile, rather than a loop without end
+            n_live = KT;
+            tile_list = 0xfedcba9876543210ull;
+        }
     } else {
         if (mask != nullptr && skip_masked_tiles) {
             const uint32_t *words = reinterpret_cast<const uint32_t *>(mask + (size_t) b * S);
