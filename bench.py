@@ -56,41 +56,41 @@ TRAFFIC_SOURCE = {  # kernel kind -> (source file under cubert_amd/csrc/kernels,
     "mask_scale_softmax": ("softmax.hip", "90a529eac55169fa"),
     "mean_pool": ("elementwise.hip", "59dcc33f61344079"),
     "classifier_head": ("elementwise.hip", "59dcc33f61344079"),
-    "attention_fused": ("attention.hip", "f321b185290e9be1"),
+    "attention_fused": ("attention.hip", "4d44df3fda986cf4"),
 }
 MEASURED_TRAFFIC = {
     "C1": {
-        "embed_ln": 25327943,
-        "attention_fused": 50081939,
-        "bias_res_ln": 37631180,
-        "bias_gelu": 100340690,
+        "embed_ln": 25327911,
+        "attention_fused": 50081728,
+        "bias_res_ln": 37631154,
+        "bias_gelu": 100340722,
         "classifier_head": 934418,
-        "mask_scale_softmax": 12589830
+        "mask_scale_softmax": 12589776
     },
     "C2": {
-        "embed_ln": 12910688,
-        "attention_fused": 25138615,
-        "bias_res_ln": 18866015,
-        "bias_gelu": 50185069,
-        "mean_pool": 6325072,
+        "embed_ln": 12910635,
+        "attention_fused": 25138608,
+        "bias_res_ln": 18866021,
+        "bias_gelu": 50185067,
+        "mean_pool": 6325126,
         "classifier_head": 147249,
-        "mask_scale_softmax": 25117442
+        "mask_scale_softmax": 25117482
     },
     "C3": {
-        "embed_ln": 99752919,
-        "attention_fused": 128669232,
-        "bias_res_ln": 150207822,
-        "bias_gelu": 400908701,
-        "classifier_head": 308800,
-        "mask_scale_softmax": 801925779
+        "embed_ln": 99735269,
+        "attention_fused": 128669160,
+        "bias_res_ln": 150207501,
+        "bias_gelu": 400907313,
+        "classifier_head": 308694,
+        "mask_scale_softmax": 801925725
     },
     "C4": {
-        "embed_ln": 133771994,
-        "attention_fused": 267267591,
-        "bias_res_ln": 200189715,
-        "bias_gelu": 534518904,
+        "embed_ln": 133764546,
+        "attention_fused": 267267622,
+        "bias_res_ln": 200189416,
+        "bias_gelu": 534518936,
         "classifier_head": 1199624,
-        "mask_scale_softmax": 267503655
+        "mask_scale_softmax": 267503672
     }
 }
 
