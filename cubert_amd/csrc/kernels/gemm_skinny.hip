@@ -14,6 +14,11 @@
 // order.  When K is cut into several slices (grid.y > 1) each workgroup stores its partial tile to a
 // workspace and the last workgroup to arrive for a feature block (ticket from an atomic counter) adds the
 // slices in slice order, so the result does not depend on scheduling.
+//
+// That hand-over (partial tile written through, ticket, partial tiles read back) is 2 us of a 7-10 us kernel.
+// gemm_skinny_partials leaves it out: every workgroup stores its partial tile and is done, and the kernel that
+// consumes the Dense layer's output (bias + residual + LayerNorm, the attention core) adds the slices in the same
+// slice order while it loads its operand, which gives the same bits.
 
 #include <cstdio>
 #include <mutex>
@@ -57,7 +62,7 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
                                                                      const T *__restrict__ bias, T *__restrict__ C,
                                                                      int ldc, int M, int N, int K, float alpha,
                                                                      float *partials, int *counters,
-                                                                     int chunks_per_slice) {
+                                                                     int chunks_per_slice, int leave_partials) {
     __shared__ float red[kSkinnyWaves][32 * 32];
     constexpr int V = 16 / sizeof(T);
     const int lane = threadIdx.x & (kWave - 1);
@@ -119,6 +124,10 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
     for (int w = 0; w < kSkinnyWaves; ++w) sum += red[w][threadIdx.x];
     const bool live = token < N && m0 + f < M;
     const int slices = gridDim.y;
+    if (leave_partials) {  // (uniform) the consumer adds the slices: partials[slice][token][feature], all 32 token rows
+        partials[((size_t) blockIdx.y * 32 + token) * ((size_t) gridDim.x * 32) + m0 + f] = sum;
+        return;
+    }
     if (slices > 1) {
         // The L2 caches of the chip's dies are not coherent with each other, and a device-scope fence would
         // write back / invalidate a whole L2 per call.  Instead every access that crosses workgroups is a
@@ -217,10 +226,10 @@ int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, int packe
     do {                                                                                                             \
         if (chunks_per_slice == kSkinnyWaves) {                                                                      \
             return launch(gemm_skinny_kernel<T, GELU, PACKED, 1>, grid, block, stream, A, lda, B, ldb, bias, C, ldc, M, \
-                          N, K, alpha, partials, counters, chunks_per_slice);                                        \
+                          N, K, alpha, partials, counters, chunks_per_slice, 0);                                     \
         }                                                                                                            \
         return launch(gemm_skinny_kernel<T, GELU, PACKED, 2>, grid, block, stream, A, lda, B, ldb, bias, C, ldc, M, N, \
-                      K, alpha, partials, counters, chunks_per_slice);                                               \
+                      K, alpha, partials, counters, chunks_per_slice, 0);                                            \
     } while (0)
     if (activation == 1) {
         if (packed) CUBERT_SKINNY_LAUNCH(true, true);
@@ -229,6 +238,38 @@ int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, int packe
     if (packed) CUBERT_SKINNY_LAUNCH(false, true);
     CUBERT_SKINNY_LAUNCH(false, false);
 #undef CUBERT_SKINNY_LAUNCH
+}
+
+// The same product left as partial tiles: partials[(slice * 32 + token) * pitch + feature] holds slice `slice` of
+// sum_k A[k, feature] B[k, token] for all 32 token rows (rows from N on are zero), *slices and *pitch say how many
+// and how wide.  No alpha, bias or activation: the consumer adds the slices in slice order (0.f + p0 + p1 + ...) and
+// goes on from there, which is what gemm_skinny's last workgroup does.  Same cut as gemm_skinny for the same
+// partial_floats; nothing is launched when the problem does not fit.
+template <typename T>
+int gemm_skinny_partials(int M, int N, int K, const T *A, int lda, int packed, const T *B, int ldb, float *partials,
+                         size_t partial_floats, int *slices_out, int *pitch_out, hipStream_t stream) {
+    if (!A || !B || !partials || !slices_out || !pitch_out) return CUBERT_BAD_ARGUMENT;
+    SkinnyPlan plan;
+    const int rc = gemm_skinny_plan<T>(M, N, K, A, lda, packed, B, ldb, M, 0, partial_floats, 0x7fffffff, &plan);
+    if (rc) return rc;
+    if ((size_t) plan.slices * 32 * plan.blocks * 32 > partial_floats) return CUBERT_UNSUPPORTED;
+    const int chunks_per_slice = plan.chunks_per_slice;
+    const dim3 grid(plan.blocks, plan.slices), block(kSkinnyThreads);
+    *slices_out = plan.slices;
+    *pitch_out = plan.blocks * 32;
+    const T *no_bias = nullptr;
+    T *no_output = nullptr;
+    int *no_counters = nullptr;
+#define CUBERT_SKINNY_PARTIALS(PACKED, PASSES)                                                                       \
+    return launch(gemm_skinny_kernel<T, false, PACKED, PASSES>, grid, block, stream, A, lda, B, ldb, no_bias, no_output, \
+                  M, M, N, K, 1.f, partials, no_counters, chunks_per_slice, 1)
+    if (chunks_per_slice == kSkinnyWaves) {
+        if (packed) CUBERT_SKINNY_PARTIALS(true, 1);
+        CUBERT_SKINNY_PARTIALS(false, 1);
+    }
+    if (packed) CUBERT_SKINNY_PARTIALS(true, 2);
+    CUBERT_SKINNY_PARTIALS(false, 2);
+#undef CUBERT_SKINNY_PARTIALS
 }
 
 // Elements of the packed form of an [K, M] weight matrix.
@@ -332,6 +373,10 @@ template int gemm_skinny<float>(int, int, int, float, const float *, int, int, c
                                 const float *, int, float *, size_t, int *, int, hipStream_t);
 template int gemm_skinny<half_t>(int, int, int, float, const half_t *, int, int, const half_t *, int, half_t *, int,
                                  const half_t *, int, float *, size_t, int *, int, hipStream_t);
+template int gemm_skinny_partials<float>(int, int, int, const float *, int, int, const float *, int, float *, size_t, int *,
+                                         int *, hipStream_t);
+template int gemm_skinny_partials<half_t>(int, int, int, const half_t *, int, int, const half_t *, int, float *, size_t,
+                                          int *, int *, hipStream_t);
 template int gemm_skinny_pack<float>(const float *, int, int, int, float *, hipStream_t);
 template int gemm_skinny_pack<half_t>(const half_t *, int, int, int, half_t *, hipStream_t);
 

@@ -127,6 +127,99 @@ __global__ __launch_bounds__(kBlock) void bias_res_ln_kernel(T *__restrict__ ino
                               split_scale, overflow);
 }
 
+// N consecutive floats (N = 2, 4 or 8) with 16-byte loads where N allows.
+template <int N>
+__device__ __forceinline__ void load_floats(const float *__restrict__ p, float (&out)[N]) {
+    if constexpr (N <= 4) {
+        const Vec<float, N> x = load_vec<float, N>(p);
+#pragma unroll
+        for (int i = 0; i < N; ++i) out[i] = x.v[i];
+    } else {
+        static_assert(N % 4 == 0, "whole 16-byte pieces");
+#pragma unroll
+        for (int q = 0; q < N / 4; ++q) {
+            const Vec<float, 4> x = load_vec<float, 4>(p + q * 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[q * 4 + i] = x.v[i];
+        }
+    }
+}
+
+// bias + residual + LayerNorm of a Dense layer that the few-token GEMM left as K slices
+// (partials[(slice * 32 + row) * pitch + col], fp32): the slices are added here, in slice order from 0.f, and the
+// sum is rounded to the storage type before anything else happens to it -- the value the GEMM's own last workgroup
+// would have stored -- so the result has the bits of GEMM followed by bias_res_ln.  At most 32 rows.
+template <typename T, int VEC, int CHUNKS, bool HAS_BIAS>
+__global__ __launch_bounds__(kBlock) void bias_res_ln_partials_kernel(T *__restrict__ out,
+                                                                      const float *__restrict__ partials, int slices,
+                                                                      int pitch, const T *__restrict__ residual,
+                                                                      const T *__restrict__ bias,
+                                                                      const T *__restrict__ beta,
+                                                                      const T *__restrict__ gamma, int rows) {
+    constexpr int H = kWave * VEC * CHUNKS;
+    constexpr int kAhead = CHUNKS * VEC <= 12 ? 8 : 4;  // slices whose loads are in flight together
+    const int row = blockIdx.x * kRowsPerBlock + wave_in_block();
+    if (row >= rows) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const float *prow = partials + (size_t) row * pitch;
+    const size_t slice_stride = (size_t) 32 * pitch;
+    const T *res = residual + (size_t) row * H;
+
+    Vec<T, VEC> r[CHUNKS], bi[CHUNKS], g[CHUNKS], be[CHUNKS];
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) r[c] = load_vec<T, VEC>(res + (c * kWave + lane) * VEC);
+    float acc[CHUNKS][VEC];
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[c][i] = 0.f;
+    }
+    for (int s0 = 0; s0 < slices; s0 += kAhead) {
+        // a slice past the last one is read from slice 0 (a valid address, so the loads go out back to back) and
+        // counted as zero
+        float p[kAhead][CHUNKS][VEC];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int s = s0 + u < slices ? s0 + u : 0;
+#pragma unroll
+            for (int c = 0; c < CHUNKS; ++c) load_floats<VEC>(prow + s * slice_stride + (c * kWave + lane) * VEC, p[u][c]);
+        }
+        if (s0 == 0) {
+#pragma unroll
+            for (int c = 0; c < CHUNKS; ++c) {
+                const int col = (c * kWave + lane) * VEC;
+                if (HAS_BIAS) bi[c] = load_vec<T, VEC>(bias + col);
+                g[c] = load_vec<T, VEC>(gamma + col);
+                be[c] = load_vec<T, VEC>(beta + col);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const bool inside = s0 + u < slices;
+#pragma unroll
+            for (int c = 0; c < CHUNKS; ++c) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc[c][i] += inside ? p[u][c][i] : 0.f;
+            }
+        }
+    }
+    float x[CHUNKS][VEC];
+    float sum = 0.f, sumsq = 0.f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            float v = to_f32(from_f32<T>(acc[c][i]));  // what the GEMM would have stored
+            if (HAS_BIAS) v += to_f32(bi[c].v[i]);
+            v += to_f32(r[c].v[i]);
+            x[c][i] = v;
+            sum += v;
+            sumsq += v * v;
+        }
+    }
+    ln_finish<T, VEC, CHUNKS>(x, sum, sumsq, g, be, out + (size_t) row * H, lane);
+}
+
 template <typename T, int VEC, int CHUNKS>
 __global__ __launch_bounds__(kBlock) void embed_ln_kernel(const int32_t *__restrict__ ids,
                                                           const int8_t *__restrict__ segments,
@@ -385,6 +478,38 @@ int bias_res_ln(T *inout, const T *residual, const T *bias, const T *beta, const
                   nullptr, beta, gamma, rows, hidden, 1);
 }
 
+// bias + residual + LayerNorm reading the Dense output as the few-token GEMM's K slices; only the register-resident
+// shapes of bias_res_ln, anything else is declined and nothing is launched.
+template <typename T>
+int bias_res_ln_partials(T *out, const float *partials, int slices, int pitch, const T *residual, const T *bias,
+                         const T *beta, const T *gamma, int rows, int hidden, void *stream) {
+    if (rows < 0 || hidden <= 0 || slices <= 0 || !out || !partials || !residual || !beta || !gamma) {
+        return CUBERT_BAD_ARGUMENT;
+    }
+    if (rows > 32 || pitch < hidden || pitch % 4 != 0 || !is_aligned(partials, 16)) return CUBERT_UNSUPPORTED;
+    if (rows == 0) return 0;
+    hipStream_t s = (hipStream_t) stream;
+    dim3 grid((rows + kRowsPerBlock - 1) / kRowsPerBlock), block(kBlock);
+    constexpr int V = MaxVec<T>::value;
+#define CUBERT_LN_CASE(VEC, CHUNKS)                                                                              \
+    if (hidden == kWave * VEC * CHUNKS && vector_ok<T>(hidden, VEC, {out, residual, bias, beta, gamma})) {       \
+        if (bias != nullptr)                                                                                     \
+            return launch(bias_res_ln_partials_kernel<T, VEC, CHUNKS, true>, grid, block, s, out, partials, slices, \
+                          pitch, residual, bias, beta, gamma, rows);                                             \
+        return launch(bias_res_ln_partials_kernel<T, VEC, CHUNKS, false>, grid, block, s, out, partials, slices, \
+                      pitch, residual, bias, beta, gamma, rows);                                                 \
+    }
+    CUBERT_LN_CASE(V, 1)
+    CUBERT_LN_CASE(V, 2)
+    CUBERT_LN_CASE(V, 3)
+    CUBERT_LN_CASE(V, 4)
+    CUBERT_LN_CASE(V / 2, 1)
+    CUBERT_LN_CASE(V / 2, 3)
+    CUBERT_LN_CASE(V / 2, 5)
+#undef CUBERT_LN_CASE
+    return CUBERT_UNSUPPORTED;
+}
+
 // bias + residual + LayerNorm of fp32 rows, in place, and the result again as two-term fp16 rows in split_out
 // [rows, 3 * hidden]; only the register-resident shapes (hidden = 256 k), anything else is declined.
 int bias_res_ln_split3(float *inout, const float *residual, const float *bias, const float *beta, const float *gamma,
@@ -474,6 +599,22 @@ extern "C" int cubert_bias_res_ln_f16(cubert_half *inout, const cubert_half *res
                                       void *stream) {
     return cubert::bias_res_ln<half_t>((half_t *) inout, (const half_t *) residual, (const half_t *) bias,
                                        (const half_t *) beta, (const half_t *) gamma, rows, hidden, stream);
+}
+
+extern "C" int cubert_bias_res_ln_partials_f32(float *out, const float *partials, int slices, int pitch,
+                                               const float *residual, const float *bias, const float *beta,
+                                               const float *gamma, int rows, int hidden, void *stream) {
+    return cubert::bias_res_ln_partials<float>(out, partials, slices, pitch, residual, bias, beta, gamma, rows, hidden,
+                                               stream);
+}
+
+extern "C" int cubert_bias_res_ln_partials_f16(cubert_half *out, const float *partials, int slices, int pitch,
+                                               const cubert_half *residual, const cubert_half *bias,
+                                               const cubert_half *beta, const cubert_half *gamma, int rows, int hidden,
+                                               void *stream) {
+    return cubert::bias_res_ln_partials<half_t>((half_t *) out, partials, slices, pitch, (const half_t *) residual,
+                                                (const half_t *) bias, (const half_t *) beta, (const half_t *) gamma,
+                                                rows, hidden, stream);
 }
 
 extern "C" int cubert_embed_ln_f32(const int32_t *ids, const int8_t *segments, const float *word, const float *pos,

@@ -32,6 +32,9 @@ int gemm_skinny_noalloc_f32(int M, int N, int K, float alpha, const float *A, in
                             int ldc, const float *bias, int activation, hipStream_t stream);
 template <typename T>
 int gemm_skinny_pack(const T *A, int lda, int M, int K, T *packed, hipStream_t stream);
+template <typename T>
+int gemm_skinny_partials(int M, int N, int K, const T *A, int lda, int packed, const T *B, int ldb, float *partials,
+                         size_t partial_floats, int *slices, int *pitch, hipStream_t stream);
 // kernels/gemm_batch.hip
 template <typename T>
 int gemm_batch(int transA, int transB, int M, int N, int K, float alpha, const T *const *A_array, int lda,
@@ -654,6 +657,31 @@ int cubert_gemm_skinny_packed_f16(void *handle, int M, int N, int K, float alpha
     if (!ctx || !packedA || !B || !C) return CUBERT_BAD_ARGUMENT;
     if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;
     return run_skinny_locked(ctx, 1, M, N, K, alpha, packedA, 0, B, ldb, C, ldc, bias, activation, 1);
+}
+
+int cubert_gemm_skinny_partials_f32(void *handle, int M, int N, int K, const float *A, int lda, int packed,
+                                    const float *B, int ldb, float *partials, size_t partial_floats, int *slices,
+                                    int *pitch) {
+    BlasContext *ctx = (BlasContext *) handle;
+    if (!ctx || !A || !B || !partials || !slices || !pitch) return CUBERT_BAD_ARGUMENT;
+    if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    ctx->used = true;
+    return cubert::gemm_skinny_partials<float>(M, N, K, A, lda, packed, B, ldb, partials, partial_floats, slices, pitch,
+                                               ctx->stream);
+}
+
+int cubert_gemm_skinny_partials_f16(void *handle, int M, int N, int K, const cubert_half *A, int lda, int packed,
+                                    const cubert_half *B, int ldb, float *partials, size_t partial_floats, int *slices,
+                                    int *pitch) {
+    BlasContext *ctx = (BlasContext *) handle;
+    if (!ctx || !A || !B || !partials || !slices || !pitch) return CUBERT_BAD_ARGUMENT;
+    if (library_gemm_only() || force_naive_gemm()) return CUBERT_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(ctx->mutex);
+    ctx->used = true;
+    return cubert::gemm_skinny_partials<cubert::half_t>(M, N, K, (const cubert::half_t *) A, lda, packed,
+                                                        (const cubert::half_t *) B, ldb, partials, partial_floats,
+                                                        slices, pitch, ctx->stream);
 }
 
 int cubert_gemm_strided_batch_f32(void *handle, int transA, int transB, int M, int N, int K, float alpha,

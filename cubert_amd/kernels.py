@@ -2,6 +2,8 @@
 and stream here): thin wrappers over the C ABI of include/cubert_kernels.h.
 Tensors must be contiguous CUDA tensors of dtype float32 or float16; kernels run
 on torch's current stream."""
+import ctypes
+
 import torch
 
 from ._lib import lib
@@ -59,6 +61,34 @@ def bias_res_ln_(inout, residual, bias, beta, gamma):
     _call("cubert_bias_res_ln", inout, _ptr(inout), _ptr(residual), _ptr(bias), _ptr(beta), _ptr(gamma), rows, hidden,
           _stream())
     return inout
+
+
+def bias_res_ln_partials(partials, residual, bias, beta, gamma):
+    """LayerNorm(storage type of (sum of the K slices partials[s, :rows, :hidden]) + bias + residual); None when the
+    shape does not fit."""
+    rows, hidden = residual.numel() // residual.shape[-1], residual.shape[-1]
+    out = torch.empty_like(residual)
+    fn = getattr(lib(), "cubert_bias_res_ln_partials_" + _suffix(residual))
+    rc = fn(_ptr(out), _ptr(partials), partials.shape[0], partials.shape[2], _ptr(residual), _ptr(bias), _ptr(beta),
+            _ptr(gamma), rows, hidden, _stream())
+    if rc == -2:
+        return None
+    _check(rc, fn.__name__)
+    return out
+
+
+def attention_partials(partials, bias, mask, heads, seq, head_size, alpha):
+    """attention_fused for one sequence whose Q|K|V projection is the K slices partials[s, 32, pitch]; bias [3 hidden]
+    in the storage type, which is also the type of the result.  None when the shape does not fit."""
+    hidden = heads * head_size
+    ctx = torch.empty((seq, hidden), dtype=bias.dtype, device=bias.device)
+    fn = getattr(lib(), "cubert_attention_partials_" + _suffix(bias))
+    rc = fn(_ptr(partials), partials.shape[0], partials.shape[2], _ptr(bias), _ptr(mask), _ptr(ctx), hidden,
+            float(alpha), heads, seq, head_size, _stream())
+    if rc == -2:
+        return None
+    _check(rc, fn.__name__)
+    return ctx
 
 
 def bias_gelu_(inout, bias):
@@ -283,6 +313,18 @@ class Blas(object):
             return None
         _check(rc, fn.__name__)
         return C
+
+    def gemm_skinny_partials(self, M, N, K, A, lda, B, ldb, packed=False, partial_floats=1 << 20):
+        """A B left as K slices: (partials[slices, 32, pitch] fp32, slices, pitch); None when the problem does not fit."""
+        partials = torch.empty(partial_floats, dtype=torch.float32, device=B.device)
+        slices, pitch = ctypes.c_int(0), ctypes.c_int(0)
+        fn = getattr(lib(), "cubert_gemm_skinny_partials_" + _suffix(B))
+        rc = fn(self.handle, M, N, K, _ptr(A), lda, int(packed), _ptr(B), ldb, _ptr(partials), partial_floats,
+                ctypes.byref(slices), ctypes.byref(pitch))
+        if rc == -2:
+            return None
+        _check(rc, fn.__name__)
+        return partials[:slices.value * 32 * pitch.value].view(slices.value, 32, pitch.value), slices.value, pitch.value
 
     def gemm_strided_batch(self, transA, transB, M, N, K, alpha, A, lda, sA, B, ldb, sB, beta, C, ldc, sC, batch):
         _call("cubert_gemm_strided_batch", C, self.handle, int(transA), int(transB), M, N, K, float(alpha), _ptr(A),

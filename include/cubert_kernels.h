@@ -70,6 +70,23 @@ int cubert_bias_res_ln_f16(cubert_half *inout, const cubert_half *residual, cons
                            const cubert_half *beta, const cubert_half *gamma, int rows, int hidden,
                            void *stream);
 
+/* cubert_bias_res_ln_* on a Dense output that cubert_gemm_skinny_partials_* left as K slices (at most 32 rows):
+ *   a = storage type of (0.f + partials[(0 * 32 + r) * pitch + c] + partials[(1 * 32 + r) * pitch + c] + ...)
+ *   x = a + bias + residual[r];  out[r] = beta + gamma * (x - mean) / sqrt(var + 1e-12)
+ * i.e. cubert_gemm_skinny_* (alpha 1, no bias) followed by cubert_bias_res_ln_*, without the GEMM's hand-over between
+ * workgroups: the same bits, except for 768 halves, where cubert_bias_res_ln_f16 runs a kernel that adds a row's sums
+ * in another order (same inputs to the LayerNorm, last-bit differences after it).  `out` is written only (it may be any buffer but `residual`).  Shapes the
+ * register-resident LayerNorm kernels do not take (hidden not 64 * {2,4,8} * {1..5}) return CUBERT_UNSUPPORTED
+ * and launch nothing.
+ * replaces: Dense + layer_norm_<T> of BertOutput / the attention output for a request of at most 32 tokens,
+ * reference src/cuBERT/op_att/Transformer.cpp:160-169 (op/Dense.cpp:47-57, op/LayerNorm.h:5-14). */
+int cubert_bias_res_ln_partials_f32(float *out, const float *partials, int slices, int pitch, const float *residual,
+                                    const float *bias, const float *beta, const float *gamma, int rows, int hidden,
+                                    void *stream);
+int cubert_bias_res_ln_partials_f16(cubert_half *out, const float *partials, int slices, int pitch,
+                                    const cubert_half *residual, const cubert_half *bias, const cubert_half *beta,
+                                    const cubert_half *gamma, int rows, int hidden, void *stream);
+
 /* bias + GELU (erf form), in place:  x = inout[r,c] + bias[c];  inout = x * 0.5 * (1 + erf(x / sqrt 2)).
  * `bias` may be NULL.
  * replaces: gelu<T>(N, inout, stream), reference src/cuBERT/op/GELU.h:6-7 (op/GELU.cu:14-26),
@@ -125,6 +142,21 @@ int cubert_attention_fused_f32(const float *q, const float *k, const float *v, i
 int cubert_attention_fused_f16(const cubert_half *q, const cubert_half *k, const cubert_half *v, int ld,
                                const int8_t *mask, cubert_half *ctx, int ld_ctx, float alpha, int batch, int heads,
                                int seq_length, int head_size, void *stream);
+
+/* cubert_attention_fused_* for ONE sequence of 32 tokens at head size 64 whose Q|K|V projection
+ * cubert_gemm_skinny_partials_* left as K slices (Q, K, V at columns 0, hidden, 2 * hidden of each partial row,
+ * hidden = heads * 64): an operand element is the storage-type rounding of (0.f + slice 0 + slice 1 + ...) + bias,
+ * the value cubert_gemm_skinny_* would have stored, so ctx has the bits of that GEMM followed by
+ * cubert_attention_fused_*.  bias: [3 * hidden], 16-byte aligned.  At most 4 slices; any other shape returns
+ * CUBERT_UNSUPPORTED and launches nothing.
+ * replaces: the Q/K/V Dense layers and the attention core of AttentionSelf<T>::_in_compute for a request of 32
+ * tokens, reference src/cuBERT/op_att/AttentionSelf.cpp:96-111. */
+int cubert_attention_partials_f32(const float *partials, int slices, int pitch, const float *bias, const int8_t *mask,
+                                  float *ctx, int ld_ctx, float alpha, int heads, int seq_length, int head_size,
+                                  void *stream);
+int cubert_attention_partials_f16(const float *partials, int slices, int pitch, const cubert_half *bias,
+                                  const int8_t *mask, cubert_half *ctx, int ld_ctx, float alpha, int heads,
+                                  int seq_length, int head_size, void *stream);
 
 /* Longest sequences first.  The long-sequence kernels (seq_length > 128) leave out key tiles (32 keys) whose mask
  * bytes are all zero, so a workgroup's time goes with its sequence's number of live tiles, and workgroups are handed
@@ -338,6 +370,25 @@ int cubert_gemm_skinny_packed_f32(void *handle, int M, int N, int K, float alpha
 int cubert_gemm_skinny_packed_f16(void *handle, int M, int N, int K, float alpha, const cubert_half *packedA,
                                   const cubert_half *B, int ldb, cubert_half *C, int ldc, const cubert_half *bias,
                                   int activation);
+
+/* The few-token product left as partial sums, for a consumer kernel that adds them while it loads its operand
+ * (cubert_bias_res_ln_partials_*, cubert_attention_partials_*).  A few-token Dense kernel spends 2 of its 7-10 us
+ * handing the K slices over to the workgroup that adds them; here every workgroup stores its slice and is done:
+ *   partials[(slice * 32 + token) * pitch + feature] = sum over the slice's k of A[k, feature] * B[k, token]
+ * for *slices slices, all 32 token rows (rows from N on are zero) and *pitch >= M features per row (fp32 whatever the
+ * storage type; no alpha, bias or activation).  Adding the slices in slice order, starting from 0.f, and rounding
+ * to the storage type gives the bits cubert_gemm_skinny_* stores for alpha = 1 and no bias.  packed != 0: A is the
+ * output of cubert_gemm_skinny_pack_* (lda ignored).  The cut is the one cubert_gemm_skinny_* makes; partials must
+ * hold partial_floats >= *slices * 32 * *pitch floats (1 << 20 is enough for every BERT-base/large Dense layer),
+ * else CUBERT_UNSUPPORTED and nothing is launched; same conditions on K, B and ldb as cubert_gemm_skinny_*.
+ * Asynchronous on the handle's stream.  No counterpart in the reference; same place as cubert_gemm_skinny_*
+ * (src/cuBERT/op/Dense.cpp:47-57). */
+int cubert_gemm_skinny_partials_f32(void *handle, int M, int N, int K, const float *A, int lda, int packed,
+                                    const float *B, int ldb, float *partials, size_t partial_floats, int *slices,
+                                    int *pitch);
+int cubert_gemm_skinny_partials_f16(void *handle, int M, int N, int K, const cubert_half *A, int lda, int packed,
+                                    const cubert_half *B, int ldb, float *partials, size_t partial_floats, int *slices,
+                                    int *pitch);
 
 /* The same over `batch_count` problems at fixed strides (in elements).
  * replaces: blas_gemm_strided_batch<T>, reference src/cuBERT/common.h:82-92. */

@@ -924,6 +924,148 @@ def test_gemm_skinny_against_oracle_sgemm(K, name, M, N, K_):
     assert_close(host(C), want, 2e-5 if name == "f32" else 2e-3, "gemm via skinny %s" % name)
 
 
+def _slices_added(partials, name):
+    """0.f + slice 0 + slice 1 + ... in fp32, rounded to the storage type: what the GEMM's last workgroup stores."""
+    total = torch.zeros_like(partials[0])
+    for s in range(partials.shape[0]):
+        total = total + partials[s]
+    return total.to(tdt(name))
+
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("M,N,K_", [(768, 32, 768), (2304, 32, 768), (768, 32, 3072), (768, 1, 768), (100, 7, 64),
+                                    (1024, 16, 4096), (3072, 20, 1024), (33, 32, 16)])
+def test_gemm_skinny_partials_add_up_to_the_gemm(K, name, packed, M, N, K_):
+    """The few-token Dense product left as K slices: added in slice order and rounded they are, bit for bit, what
+    cubert_gemm_skinny_* stores (alpha 1, no bias), rows from N on are zero, and a second product into the same
+    buffer leaves nothing of the first."""
+    rng = np.random.default_rng(M * 3 + N * 5 + K_)
+    ldb = K_ + 8
+    A = q(rng.normal(0, 1, M * K_), name)
+    blas = K.Blas()
+    dA = dev(A, tdt(name))
+    weights = blas.gemm_skinny_pack(dA, M, M, K_) if packed else dA
+    for trial in range(2):
+        B = q(rng.normal(0, 1, N * ldb), name)
+        dB = dev(B, tdt(name))
+        got = blas.gemm_skinny_partials(M, N, K_, weights, M, dB, ldb, packed=packed)
+        assert got is not None
+        partials, slices, pitch = got
+        assert pitch >= M and pitch % 32 == 0 and slices >= 1
+        C = torch.full((N * M,), 7.0, dtype=tdt(name), device="cuda")
+        if packed:
+            assert blas.gemm_skinny_packed(M, N, K_, 1.0, weights, dB, ldb, C, M) is not None
+        else:
+            assert blas.gemm_skinny(M, N, K_, 1.0, dA, M, dB, ldb, C, M) is not None
+        added = _slices_added(partials, name)
+        assert torch.equal(added[:N, :M].contiguous().view(-1), C)
+        assert not partials[:, N:, :].any()
+    want = oracle.sgemm(0, 0, M, N, K_, 1.0, A, M, B, ldb, 0.0, np.zeros(N * M, np.float32), M)
+    assert_close(host(added[:N, :M]).ravel(), want, 2e-5 if name == "f32" else 2e-3, "partials %s" % name)
+
+
+def test_gemm_skinny_partials_declines_what_it_cannot_do(K):
+    blas = K.Blas()
+    x = torch.zeros(64 * 1024, device="cuda")
+    assert blas.gemm_skinny_partials(64, 33, 64, x, 64, x, 64) is None             # more than 32 tokens
+    assert blas.gemm_skinny_partials(64, 8, 24, x, 64, x, 24) is None              # K not a multiple of 16
+    assert blas.gemm_skinny_partials(64, 8, 32, x, 64, x[1:], 32) is None          # misaligned activations
+    assert blas.gemm_skinny_partials(768, 8, 768, x, 768, x, 768, partial_floats=1000) is None  # buffer too small
+    assert blas.gemm_skinny_partials(64, 8, 32, x, 64, x, 32, partial_floats=2048) is not None
+
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("rows,hidden,in_features,with_bias", [(32, 768, 768, True), (32, 768, 3072, True),
+                                                               (7, 768, 3072, False), (1, 1024, 4096, True),
+                                                               (20, 256, 1024, True), (32, 512, 64, False)])
+def test_bias_res_ln_from_partials_has_the_bits_of_gemm_then_layer_norm(K, name, rows, hidden, in_features, with_bias):
+    rng = np.random.default_rng(rows + hidden + in_features)
+    blas = K.Blas()
+    W = dev(q(rng.normal(0, 0.05, in_features * hidden), name), tdt(name))          # [in, out]
+    X = dev(q(rng.normal(0, 1, rows * in_features), name), tdt(name))
+    residual = dev(q(rng.normal(0, 1, (rows, hidden)), name), tdt(name))
+    bias = dev(q(rng.normal(0, 1, hidden), name), tdt(name)) if with_bias else None
+    beta, gamma = (dev(q(rng.normal(0, 1, hidden), name), tdt(name)) for _ in range(2))
+    C = torch.zeros((rows, hidden), dtype=tdt(name), device="cuda")
+    assert blas.gemm_skinny(hidden, rows, in_features, 1.0, W, hidden, X, in_features, C, hidden) is not None
+    dense_values = host(C)
+    want = K.bias_res_ln_(C, residual, bias, beta, gamma)
+    partials, slices, pitch = blas.gemm_skinny_partials(hidden, rows, in_features, W, hidden, X, in_features)
+    got = K.bias_res_ln_partials(partials, residual, bias, beta, gamma)
+    assert got is not None
+    if name == "f32" or hidden != 768:
+        assert torch.equal(got, want)
+    else:
+        # 768 halves: bias_res_ln takes its two-rows-per-wavefront kernel there, whose row sums are added in another
+        # order; the values that go into the LayerNorm are the same
+        assert_close(host(got), host(want), 1e-3, "LayerNorm from partials against LayerNorm of the GEMM output")
+    # and against the oracle's LayerNorm of the values the GEMM stored
+    ref = oracle.layer_norm_(host(residual), dense_values + (host(bias) if with_bias else 0.0), host(beta), host(gamma))
+    assert_close(host(got), ref, 2e-5 if name == "f32" else 4e-3, "LayerNorm from partials %s" % name)
+
+
+def test_bias_res_ln_from_partials_declines_what_it_cannot_do(K):
+    partials = torch.zeros((3, 32, 768), device="cuda")
+    v = torch.zeros(768, device="cuda")
+    assert K.bias_res_ln_partials(partials, torch.zeros((33, 768), device="cuda"), v, v, v) is None   # 33 rows
+    narrow = torch.zeros((3, 32, 128), device="cuda")
+    assert K.bias_res_ln_partials(narrow, torch.zeros((4, 100), device="cuda"), v[:100], v[:100], v[:100]) is None  # hidden 100
+    assert K.bias_res_ln_partials(narrow, torch.zeros((4, 768), device="cuda"), v, v, v) is None  # rows narrower than hidden
+
+
+@pytest.mark.parametrize("name", ["f32", "f16"])
+@pytest.mark.parametrize("heads,masked", [(12, True), (12, False), (16, True), (2, True)])
+def test_attention_from_partials_has_the_bits_of_gemm_then_attention(K, name, heads, masked):
+    """One sequence of 32 tokens: Q|K|V projection left as K slices, attention core reading them."""
+    seq, d = 32, 64
+    hidden = heads * d
+    rng = np.random.default_rng(heads * 2 + masked)
+    blas = K.Blas()
+    W = dev(q(rng.normal(0, 0.05, hidden * 3 * hidden), name), tdt(name))          # [in, 3 * hidden]
+    X = dev(q(rng.normal(0, 1, seq * hidden), name), tdt(name))
+    bias = dev(q(rng.normal(0, 0.5, 3 * hidden), name), tdt(name))
+    mask = None
+    if masked:
+        m = np.ones(seq, np.int8)
+        m[rng.integers(5, seq):] = 0
+        m[2] = 0
+        mask = dev(m)
+    qkv = torch.zeros((seq, 3 * hidden), dtype=tdt(name), device="cuda")
+    assert blas.gemm_skinny(3 * hidden, seq, hidden, 1.0, W, 3 * hidden, X, hidden, qkv, 3 * hidden, bias=bias) is not None
+    want = K.attention_fused(qkv, mask, 1, heads, seq, d, 0.125)
+    assert want is not None
+    got = blas.gemm_skinny_partials(3 * hidden, seq, hidden, W, 3 * hidden, X, hidden)
+    assert got is not None
+    partials, slices, pitch = got
+    ctx = K.attention_partials(partials, bias, mask, heads, seq, d, 0.125)
+    assert ctx is not None
+    assert torch.equal(ctx, want)
+    # and against the oracle on the projection the GEMM stored
+    stored = host(qkv)
+    qh, kh, vh = (np.ascontiguousarray(x) for x in (stored[:, :hidden], stored[:, hidden:2 * hidden], stored[:, 2 * hidden:]))
+    scores = oracle.att_q_k(qh, kh, 1, seq, heads, d, alpha=0.125)
+    if name == "f16":
+        scores = oracle.round_to_half(scores)
+    if masked:
+        scores = scores + (-10000.0 * (1.0 - m.astype(np.float32)))[None, None, None, :]
+    p = oracle.softmax_(np.ascontiguousarray(scores.reshape(-1, seq), dtype=np.float32)).reshape(scores.shape)
+    if name == "f16":
+        p = oracle.round_to_half(p)
+    ref = oracle.att_qk_v(np.ascontiguousarray(p, dtype=np.float32), vh, 1, seq, heads, d).reshape(seq, hidden)
+    assert_close(host(ctx), ref, 2e-5 if name == "f32" else 2e-3, "attention from partials %s" % name)
+
+
+def test_attention_from_partials_declines_what_it_cannot_do(K):
+    partials = torch.zeros((3, 32, 2304), device="cuda")
+    bias = torch.zeros(2304, device="cuda")
+    assert K.attention_partials(partials, bias, None, 12, 16, 64, 0.125) is None     # not 32 tokens
+    assert K.attention_partials(partials, bias, None, 24, 32, 32, 0.125) is None     # head size 32
+    assert K.attention_partials(torch.zeros((3, 32, 2048), device="cuda"), bias, None, 12, 32, 64, 0.125) is None  # rows too narrow
+    many = torch.zeros((5, 32, 2304), device="cuda")
+    assert K.attention_partials(many, bias, None, 12, 32, 64, 0.125) is None         # more than four slices
+
+
 def test_gemm_skinny_declines_what_it_cannot_do(K):
     blas = K.Blas()
     x = torch.zeros(64 * 1024, device="cuda")
