@@ -133,7 +133,6 @@ for _t in ("f32", "f16"):
         "cubert_gemm_skinny_partials_" + _t: (ci, [vp, ci, ci, ci, vp, ci, ci, vp, ci, vp, ctypes.c_size_t,
                                                   ctypes.POINTER(ci), ctypes.POINTER(ci)]),
         "cubert_bias_res_ln_partials_" + _t: (ci, [vp, vp, ci, ci, vp, vp, vp, vp, ci, ci, vp]),
-        "cubert_attention_partials_" + _t: (ci, [vp, ci, ci, vp, vp, vp, ci, cf, ci, ci, ci, vp]),
         "cubert_gemm_strided_batch_" + _t: (ci, [vp, ci, ci, ci, ci, ci, cf, vp, ci, cll, vp, ci, cll, cf, vp, ci, cll, ci]),
         "cubert_gemm_batch_" + _t: (ci, [vp, ci, ci, ci, ci, ci, cf, vp, ci, vp, ci, cf, vp, ci, ci]),
     })

@@ -195,6 +195,7 @@ void Transformer<T>::layout_buffers() {
     layer_output[0] = buffers.take<T>(M * H);
     layer_output[1] = buffers.take<T>(M * H);
     if (split_dense) split_operand = buffers.take<half>(M * 3 * (H > intermediate_size ? H : intermediate_size));
+    if (seq_length <= 32) few_token_partials = buffers.take<float>(kFewTokenPartialFloats);
 }
 
 template <typename T>
@@ -336,6 +337,45 @@ void Transformer<T>::dense_split(int out_features, int tokens, int in_features, 
     }
 }
 
+// CUBERT_FEW_TOKEN_SLICES=0 in the environment keeps the few-token Dense kernels adding their own K slices.
+static bool few_token_slices_enabled() {
+    static const bool on = [] {
+        const char *e = std::getenv("CUBERT_FEW_TOKEN_SLICES");
+        return e == nullptr || std::string(e) != "0";
+    }();
+    return on;
+}
+
+template <typename T>
+void Transformer<T>::dense_norm(int tokens, int in_features, const T *kernel, const T *packed, const T *in, const T *bias,
+                                const T *residual, const T *beta, const T *gamma, T *out, Profiler::Kind kind) {
+    void *stream = cuBERT::blas_get_stream(cublas);
+    const int H = (int) hidden_size;
+    if (tokens <= 32 && slices_to_norm && few_token_partials != nullptr && few_token_slices_enabled() &&
+        (packed != nullptr || !transposed_kernels)) {
+        int slices = 0, pitch = 0;
+        bool done = false;
+        {
+            Timed t(profiler, profiler != nullptr ? profiler->dense_kind(kind) : Profiler::kDenseGemm, stream);
+            done = cuBERT::dense_few_tokens_partials(cublas, H, tokens, in_features, kernel, H, packed, in, in_features,
+                                                     few_token_partials, kFewTokenPartialFloats, &slices, &pitch);
+            if (!done) t.cancel();
+        }
+        if (done) {
+            Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
+            if (cuBERT::layer_norm_partials(out, few_token_partials, slices, pitch, residual, bias, beta, gamma, tokens, H,
+                                            stream)) {
+                return;
+            }
+            t.cancel();
+        }
+        slices_to_norm = false;  // the layer sizes are fixed per model: do not ask again
+    }
+    const bool bias_done = dense(H, tokens, in_features, kernel, packed, in, out, bias, false, false, kind);
+    Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
+    cuBERT::layer_norm_(residual, out, tokens, H, bias_done ? nullptr : bias, beta, gamma, stream);
+}
+
 template <typename T>
 T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attention_mask) {
     if (batch_size > max_batch_size) throw std::invalid_argument("batch_size > max_batch_size");
@@ -413,14 +453,9 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
         attention(batch_size, qkv_out, attention_mask);
 
         // attention/output: dense, then bias + residual(layer input) + LayerNorm
-        const bool ao_bias = dense(H, M, H, w.attention_output_kernel, w.attention_output_packed, context_out,
-                                   attention_output, w.attention_output_bias, false, false,
-                                   Profiler::kDenseAttentionOutput);
-        {
-            Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
-            cuBERT::layer_norm_(layer_input, attention_output, M, H, ao_bias ? nullptr : w.attention_output_bias,
-                                w.attention_norm_beta, w.attention_norm_gamma, stream);
-        }
+        dense_norm(M, H, w.attention_output_kernel, w.attention_output_packed, context_out, w.attention_output_bias,
+                   layer_input, w.attention_norm_beta, w.attention_norm_gamma, attention_output,
+                   Profiler::kDenseAttentionOutput);
 
         // intermediate: dense, then bias + GELU (one launch for all three at <= 32 tokens)
         if (!dense(I, M, H, w.intermediate_kernel, w.intermediate_packed, attention_output, intermediate_output,
@@ -430,13 +465,8 @@ T *Transformer<T>::_in_compute(size_t batch_size, T *input_gpu, int8_t *attentio
         }
 
         // output: dense, then bias + residual(attention output) + LayerNorm
-        const bool out_bias = dense(H, M, I, w.output_kernel, w.output_packed, intermediate_output, out, w.output_bias,
-                                    false, false, Profiler::kDenseOutput);
-        {
-            Timed t(profiler, Profiler::kBiasResLayerNorm, stream);
-            cuBERT::layer_norm_(attention_output, out, M, H, out_bias ? nullptr : w.output_bias, w.output_norm_beta,
-                                w.output_norm_gamma, stream);
-        }
+        dense_norm(M, I, w.output_kernel, w.output_packed, intermediate_output, w.output_bias, attention_output,
+                   w.output_norm_beta, w.output_norm_gamma, out, Profiler::kDenseOutput);
 
         prev_output = out;
     }

@@ -3,7 +3,8 @@
 // named-weight map under a variable prefix, then compute(batch, input, mask)
 // with device pointers, returning a device pointer to [batch, seq, hidden].
 //
-// Inside, a layer is 8 launches (7 for at most 32 tokens):
+// Inside, a layer is 8 launches (7 for at most 32 tokens, where the two Dense kernels in front of a LayerNorm also
+// leave their K slices to it instead of adding them up themselves):
 //   qkv   = x * [Wq|Wk|Wv] + [bq|bk|bv]          one GEMM, bias in its epilogue
 //   ctx   = softmax((1/sqrt d) Q K^T + mask) V    one attention kernel (scores stay in registers); where its
 //                                                 shape limits do not hold: scores kernel or batched GEMM into
@@ -111,9 +112,15 @@ private:
     // split_operand first, or, when null, split_operand already holds the [hi | hi | lo] rows.  `bias` may be null.
     void dense_split(int out_features, int tokens, int in_features, const SplitKernel &kernel, const T *in, T *out,
                      const T *bias, Profiler::Kind kind, int ld_out = 0);
+    // out = LayerNorm(in * kernel + bias + residual): dense(), then layer_norm_; for at most 32 tokens the few-token
+    // GEMM leaves its K slices in few_token_partials and the LayerNorm kernel adds them while it loads (same values,
+    // without the GEMM's 2 us hand-over between workgroups).
+    void dense_norm(int tokens, int in_features, const T *kernel, const T *packed, const T *in, const T *bias,
+                    const T *residual, const T *beta, const T *gamma, T *out, Profiler::Kind kind);
 
     void *cublas;
     Profiler *profiler = nullptr;
+    bool slices_to_norm = true;        // few-token Dense layers hand their K slices to the LayerNorm (cleared when declined)
     bool dense_gelu_fits = true;       // cleared when the few-token Dense + GELU kernel declines this model's shape
     bool keep_packed = false;          // Dense kernels are also kept in the few-token kernel's order
     bool transposed_kernels = false;   // Dense kernels are stored [out, in] instead of [in, out] (half precision)
@@ -139,6 +146,8 @@ private:
     T *intermediate_output;  // [M, intermediate]
     T *layer_output[2];      // [M, hidden], alternating between layers
     half *split_operand = nullptr;  // [M, 3 * max(hidden, intermediate)] two-term rows of the current Dense input
+    static constexpr size_t kFewTokenPartialFloats = (size_t) 1 << 20;
+    float *few_token_partials = nullptr;  // K slices of the current few-token Dense layer (seq_length <= 32 only)
 };
 
 }  // namespace cuBERT

@@ -102,6 +102,45 @@ inline bool dense_few_tokens(void *handle, int M, int N, int K, const half *A, i
     CUBERT_CHECK(rc);
     return true;
 }
+// The same product left as K slices for the kernel that consumes it (layer_norm_partials):
+// partials[(slice * 32 + token) * pitch + feature], fp32; false when the kernel does not take the problem.
+inline bool dense_few_tokens_partials(void *handle, int M, int N, int K, const float *A, int lda, const float *packed,
+                                      const float *B, int ldb, float *partials, size_t partial_floats, int *slices,
+                                      int *pitch) {
+    const int rc = cubert_gemm_skinny_partials_f32(handle, M, N, K, packed ? packed : A, lda, packed != nullptr, B, ldb,
+                                                   partials, partial_floats, slices, pitch);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+inline bool dense_few_tokens_partials(void *handle, int M, int N, int K, const half *A, int lda, const half *packed,
+                                      const half *B, int ldb, float *partials, size_t partial_floats, int *slices,
+                                      int *pitch) {
+    const int rc = cubert_gemm_skinny_partials_f16(handle, M, N, K, h(packed ? packed : A), lda, packed != nullptr, h(B),
+                                                   ldb, partials, partial_floats, slices, pitch);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+// out = LayerNorm(storage type of (sum of the slices) + bias + residual) for at most 32 rows; false when declined
+inline bool layer_norm_partials(float *out, const float *partials, int slices, int pitch, const float *residual,
+                                const float *bias, const float *beta, const float *gamma, int rows, int hidden,
+                                void *stream) {
+    const int rc = cubert_bias_res_ln_partials_f32(out, partials, slices, pitch, residual, bias, beta, gamma, rows,
+                                                   hidden, stream);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
+inline bool layer_norm_partials(half *out, const float *partials, int slices, int pitch, const half *residual,
+                                const half *bias, const half *beta, const half *gamma, int rows, int hidden,
+                                void *stream) {
+    const int rc = cubert_bias_res_ln_partials_f16(h(out), partials, slices, pitch, h(residual), h(bias), h(beta),
+                                                   h(gamma), rows, hidden, stream);
+    if (rc == CUBERT_UNSUPPORTED) return false;
+    CUBERT_CHECK(rc);
+    return true;
+}
 inline void pack_few_token_weights(void *handle, const float *A, int lda, int M, int K, float *packed) {
     CUBERT_CHECK(cubert_gemm_skinny_pack_f32(handle, A, lda, M, K, packed));
 }

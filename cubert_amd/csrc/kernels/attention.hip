@@ -742,59 +742,12 @@ __global__ __launch_bounds__(KT * kWave) void attention_fused_half_kernel(const 
 // used by one lane only), the four partial score tiles are added in wavefront order through LDS, every
 // wavefront repeats the (cheap) softmax, and P V is split into (column tile, key half), the two key halves
 // meeting in LDS again.  Same arithmetic and rounding as attention_fused_kernel, other summation order.
-//
-// PARTIALS: the Q|K|V projection arrives as the K slices the few-token GEMM left (PartialSource), and an operand
-// element is the storage-type rounding of (0.f + slice 0 + slice 1 + ...) + bias -- what that GEMM's last workgroup
-// would have stored -- so the result has the bits of GEMM followed by this kernel.  One sequence (batch 1) only: the
-// slices hold 32 token rows.
-struct PartialSource {
-    const float *data = nullptr;  // [slice][32 tokens][pitch] with Q, K, V at columns 0, hidden, 2 * hidden
-    int slices = 0, pitch = 0, hidden = 0;
-    const void *bias = nullptr;   // [3 * hidden] in the storage type
-};
-constexpr int kAttentionPartialSlices = 4;  // slices a lane's operand loads are unrolled over
-
-// `width` consecutive operand elements starting at column `col` of token row `row`.
-template <typename T, int W>
-__device__ __forceinline__ Vec<T, W> partial_operand(const PartialSource &src, int row, int col) {
-    static_assert(W == 1 || W % 4 == 0, "whole 16-byte pieces of floats, or one element");
-    float sum[W];
-#pragma unroll
-    for (int e = 0; e < W; ++e) sum[e] = 0.f;
-    float part[kAttentionPartialSlices][W];
-#pragma unroll
-    for (int s = 0; s < kAttentionPartialSlices; ++s) {
-        // (a slice past the last is read from slice 0, a valid address, and counted as zero)
-        const float *at = src.data + ((size_t) (s < src.slices ? s : 0) * 32 + row) * src.pitch + col;
-        if constexpr (W == 1) {
-            part[s][0] = *at;
-        } else {
-#pragma unroll
-            for (int q4 = 0; q4 < W / 4; ++q4) {
-                const Vec<float, 4> x = load_vec<float, 4>(at + q4 * 4);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) part[s][q4 * 4 + e] = x.v[e];
-            }
-        }
-    }
-    const Vec<T, W> b = load_vec<T, W>(static_cast<const T *>(src.bias) + col);
-#pragma unroll
-    for (int s = 0; s < kAttentionPartialSlices; ++s) {
-#pragma unroll
-        for (int e = 0; e < W; ++e) sum[e] += s < src.slices ? part[s][e] : 0.f;
-    }
-    Vec<T, W> out;
-#pragma unroll
-    for (int e = 0; e < W; ++e) out.v[e] = from_f32<T>(sum[e] + to_f32(b.v[e]));
-    return out;
-}
-
-template <typename T, bool SPLIT, bool PARTIALS = false>
+template <typename T, bool SPLIT>
 __global__ __launch_bounds__(4 * kWave) void attention_small_kernel(const T *__restrict__ q, const T *__restrict__ k,
                                                                     const T *__restrict__ v, int ld,
                                                                     const int8_t *__restrict__ mask,
                                                                     T *__restrict__ ctx, int ld_ctx, float alpha,
-                                                                    int heads, SplitOut split, PartialSource src) {
+                                                                    int heads, SplitOut split) {
     constexpr int D = 64, S = 32;
     constexpr int V = Mma<T>::kVec;
     constexpr int kSteps = D / 8 / V;  // operand vectors per lane and contraction: a quarter of D over two lane halves
@@ -811,23 +764,14 @@ __global__ __launch_bounds__(4 * kWave) void attention_small_kernel(const T *__r
     Vec<T, V> qv[kSteps], kv[kSteps];
 #pragma unroll
     for (int t = 0; t < kSteps; ++t) {
-        if constexpr (PARTIALS) {
-            qv[t] = partial_operand<T, V>(src, r, (int) d0 + t * V);
-            kv[t] = partial_operand<T, V>(src, r, src.hidden + (int) d0 + t * V);
-        } else {
-            qv[t] = load_vec<T, V>(q + (row0 + r) * ld + d0 + t * V);
-            kv[t] = load_vec<T, V>(k + (row0 + r) * ld + d0 + t * V);
-        }
+        qv[t] = load_vec<T, V>(q + (row0 + r) * ld + d0 + t * V);
+        kv[t] = load_vec<T, V>(k + (row0 + r) * ld + d0 + t * V);
     }
     const int jt = w & 1, kh = w >> 1;  // second contraction: output columns jt*32 .. +31, keys of registers kh*8 .. +7
     T vreg[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        if constexpr (PARTIALS) {
-            vreg[i] = partial_operand<T, 1>(src, acc_row(kh * 8 + i, hh), 2 * src.hidden + h * D + jt * 32 + r).v[0];
-        } else {
-            vreg[i] = v[(row0 + acc_row(kh * 8 + i, hh)) * ld + (size_t) h * D + jt * 32 + r];
-        }
+        vreg[i] = v[(row0 + acc_row(kh * 8 + i, hh)) * ld + (size_t) h * D + jt * 32 + r];
     }
     float add[16];  // additive mask of this lane's 16 keys, in units of log 2
 #pragma unroll
@@ -1587,12 +1531,12 @@ int launch_fused(const T *q, const T *k, const T *v, int ld, const int8_t *mask,
             if constexpr (sizeof(T) == 4) {
                 if (split.width > 0) {
                     return launch_lds(attention_small_kernel<T, true>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q,
-                                          k, v, ld, mask, ctx, ld_ctx, alpha, heads, split, PartialSource{});
+                                          k, v, ld, mask, ctx, ld_ctx, alpha, heads, split);
                 }
             }
             if (split.width > 0) return CUBERT_UNSUPPORTED;
             return launch_lds(attention_small_kernel<T, false>, dim3(batch * heads), dim3(4 * kWave), 0u, s, q, k, v,
-                                  ld, mask, ctx, ld_ctx, alpha, heads, split, PartialSource{});
+                                  ld, mask, ctx, ld_ctx, alpha, heads, split);
         }
     }
     switch (seq / 32) {
@@ -1689,25 +1633,6 @@ int attention_fused(const T *q, const T *k, const T *v, int ld, const int8_t *ma
     }
 }
 
-
-// The attention core of ONE sequence of 32 tokens (head size 64) whose Q|K|V projection the few-token GEMM left as
-// K slices; anything else is declined and nothing is launched.
-template <typename T>
-int attention_partials(const float *partials, int slices, int pitch, const T *bias, const int8_t *mask, T *ctx,
-                       int ld_ctx, float alpha, int heads, int seq, int head_size, void *stream) {
-    if (!partials || !bias || !ctx || slices <= 0 || heads <= 0 || seq <= 0 || head_size <= 0) return CUBERT_BAD_ARGUMENT;
-    const int hidden = heads * head_size;
-    if (seq != 32 || head_size != 64 || slices > kAttentionPartialSlices || pitch < 3 * hidden || pitch % 4 != 0 ||
-        ld_ctx < hidden || !is_aligned(partials, 16) || !is_aligned(bias, 16) ||
-        (mask != nullptr && !is_aligned(mask, 4))) {
-        return CUBERT_UNSUPPORTED;
-    }
-    PartialSource src;
-    src.data = partials, src.slices = slices, src.pitch = pitch, src.hidden = hidden, src.bias = bias;
-    const T *none = nullptr;
-    return launch_lds(attention_small_kernel<T, false, true>, dim3(heads), dim3(4 * kWave), 0u, (hipStream_t) stream,
-                      none, none, none, 0, mask, ctx, ld_ctx, alpha, heads, SplitOut(), src);
-}
 }  // namespace
 }  // namespace cubert
 
@@ -1779,19 +1704,4 @@ extern "C" int cubert_attention_fused_f16(const cubert_half *q, const cubert_hal
     return cubert::attention_fused<cubert::half_t>((const cubert::half_t *) q, (const cubert::half_t *) k,
                                                    (const cubert::half_t *) v, ld, mask, (cubert::half_t *) ctx,
                                                    ld_ctx, alpha, batch, heads, seq_length, head_size, stream);
-}
-
-extern "C" int cubert_attention_partials_f32(const float *partials, int slices, int pitch, const float *bias,
-                                             const int8_t *mask, float *ctx, int ld_ctx, float alpha, int heads,
-                                             int seq_length, int head_size, void *stream) {
-    return cubert::attention_partials<float>(partials, slices, pitch, bias, mask, ctx, ld_ctx, alpha, heads, seq_length,
-                                             head_size, stream);
-}
-
-extern "C" int cubert_attention_partials_f16(const float *partials, int slices, int pitch, const cubert_half *bias,
-                                             const int8_t *mask, cubert_half *ctx, int ld_ctx, float alpha, int heads,
-                                             int seq_length, int head_size, void *stream) {
-    return cubert::attention_partials<cubert::half_t>(partials, slices, pitch, (const cubert::half_t *) bias, mask,
-                                                      (cubert::half_t *) ctx, ld_ctx, alpha, heads, seq_length,
-                                                      head_size, stream);
 }

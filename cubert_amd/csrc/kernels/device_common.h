@@ -51,6 +51,25 @@ __device__ __forceinline__ void split_two_terms(float x, half_t &hi, half_t &lo)
 // consumes them must be told (the kernels that write two-term rows raise a flag the caller looks at).
 __device__ __forceinline__ bool two_term_overflow(float x) { return !(fabsf(x) <= 65504.f); }
 
+// x when keep, +0.f otherwise, as a bit operation: a select between a loaded value and zero invites the compiler to
+// put the load itself under a branch, where it is waited for on the spot.
+__device__ __forceinline__ float keep_or_zero(float x, bool keep) {
+    return __builtin_bit_cast(float, __builtin_bit_cast(unsigned, x) & (keep ? 0xffffffffu : 0u));
+}
+
+// An empty statement that counts as a use and a redefinition of x (whole 32-bit registers).  Such statements keep
+// their order among themselves, and a loaded value has to have arrived before one that names it: a way to make the
+// compiler request a load early instead of where its value is first needed.
+template <typename X>
+__device__ __forceinline__ void pin_registers(X &x) {
+    static_assert(sizeof(X) % 4 == 0, "whole registers");
+    unsigned words[sizeof(X) / 4];
+    __builtin_memcpy(words, &x, sizeof(X));
+#pragma unroll
+    for (unsigned i = 0; i < sizeof(X) / 4; ++i) asm volatile("" : "+v"(words[i]));
+    __builtin_memcpy(&x, words, sizeof(X));
+}
+
 // Widest vector (in elements) that is at most 16 bytes.
 template <typename T>
 struct MaxVec {

@@ -17,8 +17,8 @@
 //
 // That hand-over (partial tile written through, ticket, partial tiles read back) is 2 us of a 7-10 us kernel.
 // gemm_skinny_partials leaves it out: every workgroup stores its partial tile and is done, and the kernel that
-// consumes the Dense layer's output (bias + residual + LayerNorm, the attention core) adds the slices in the same
-// slice order while it loads its operand, which gives the same bits.
+// consumes the Dense layer's output (bias + residual + LayerNorm) adds the slices in the same slice order while it
+// loads its operand, which gives the same bits.
 
 #include <cstdio>
 #include <mutex>

@@ -158,7 +158,7 @@ __global__ __launch_bounds__(kBlock) void bias_res_ln_partials_kernel(T *__restr
                                                                       const T *__restrict__ gamma, int rows) {
     constexpr int H = kWave * VEC * CHUNKS;
     constexpr int kAhead = CHUNKS * VEC <= 12 ? 8 : 4;  // slices whose loads are in flight together
-    const int row = blockIdx.x * kRowsPerBlock + wave_in_block();
+    const int row = blockIdx.x * (int) (blockDim.x / kWave) + wave_in_block();
     if (row >= rows) return;
     const int lane = threadIdx.x & (kWave - 1);
     const float *prow = partials + (size_t) row * pitch;
@@ -192,6 +192,14 @@ __global__ __launch_bounds__(kBlock) void bias_res_ln_partials_kernel(T *__restr
                 g[c] = load_vec<T, VEC>(gamma + col);
                 be[c] = load_vec<T, VEC>(beta + col);
             }
+            // (requested here, with the slices: the compiler would otherwise move these loads to where the values are
+            // used, behind the loop, one more memory latency at the end of the kernel)
+#pragma unroll
+            for (int c = 0; c < CHUNKS; ++c) {
+                if (HAS_BIAS) pin_registers(bi[c]);
+                pin_registers(g[c]);
+                pin_registers(be[c]);
+            }
         }
 #pragma unroll
         for (int u = 0; u < kAhead; ++u) {
@@ -199,7 +207,7 @@ __global__ __launch_bounds__(kBlock) void bias_res_ln_partials_kernel(T *__restr
 #pragma unroll
             for (int c = 0; c < CHUNKS; ++c) {
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) acc[c][i] += inside ? p[u][c][i] : 0.f;
+                for (int i = 0; i < VEC; ++i) acc[c][i] += u == 0 ? p[u][c][i] : keep_or_zero(p[u][c][i], inside);
             }
         }
     }
@@ -489,7 +497,9 @@ int bias_res_ln_partials(T *out, const float *partials, int slices, int pitch, c
     if (rows > 32 || pitch < hidden || pitch % 4 != 0 || !is_aligned(partials, 16)) return CUBERT_UNSUPPORTED;
     if (rows == 0) return 0;
     hipStream_t s = (hipStream_t) stream;
-    dim3 grid((rows + kRowsPerBlock - 1) / kRowsPerBlock), block(kBlock);
+    // a wavefront per workgroup: what a row waits for is its slices arriving, and a compute unit pulls them at a
+    // fraction of what the memory system delivers, so the rows are spread over as many compute units as there are rows
+    dim3 grid(rows), block(kWave);
     constexpr int V = MaxVec<T>::value;
 #define CUBERT_LN_CASE(VEC, CHUNKS)                                                                              \
     if (hidden == kWave * VEC * CHUNKS && vector_ok<T>(hidden, VEC, {out, residual, bias, beta, gamma})) {       \

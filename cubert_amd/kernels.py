@@ -77,20 +77,6 @@ def bias_res_ln_partials(partials, residual, bias, beta, gamma):
     return out
 
 
-def attention_partials(partials, bias, mask, heads, seq, head_size, alpha):
-    """attention_fused for one sequence whose Q|K|V projection is the K slices partials[s, 32, pitch]; bias [3 hidden]
-    in the storage type, which is also the type of the result.  None when the shape does not fit."""
-    hidden = heads * head_size
-    ctx = torch.empty((seq, hidden), dtype=bias.dtype, device=bias.device)
-    fn = getattr(lib(), "cubert_attention_partials_" + _suffix(bias))
-    rc = fn(_ptr(partials), partials.shape[0], partials.shape[2], _ptr(bias), _ptr(mask), _ptr(ctx), hidden,
-            float(alpha), heads, seq, head_size, _stream())
-    if rc == -2:
-        return None
-    _check(rc, fn.__name__)
-    return ctx
-
-
 def bias_gelu_(inout, bias):
     rows, width = inout.numel() // inout.shape[-1], inout.shape[-1]
     _call("cubert_bias_gelu", inout, _ptr(inout), _ptr(bias), rows, width, _stream())

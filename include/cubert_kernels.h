@@ -143,21 +143,6 @@ int cubert_attention_fused_f16(const cubert_half *q, const cubert_half *k, const
                                const int8_t *mask, cubert_half *ctx, int ld_ctx, float alpha, int batch, int heads,
                                int seq_length, int head_size, void *stream);
 
-/* cubert_attention_fused_* for ONE sequence of 32 tokens at head size 64 whose Q|K|V projection
- * cubert_gemm_skinny_partials_* left as K slices (Q, K, V at columns 0, hidden, 2 * hidden of each partial row,
- * hidden = heads * 64): an operand element is the storage-type rounding of (0.f + slice 0 + slice 1 + ...) + bias,
- * the value cubert_gemm_skinny_* would have stored, so ctx has the bits of that GEMM followed by
- * cubert_attention_fused_*.  bias: [3 * hidden], 16-byte aligned.  At most 4 slices; any other shape returns
- * CUBERT_UNSUPPORTED and launches nothing.
- * replaces: the Q/K/V Dense layers and the attention core of AttentionSelf<T>::_in_compute for a request of 32
- * tokens, reference src/cuBERT/op_att/AttentionSelf.cpp:96-111. */
-int cubert_attention_partials_f32(const float *partials, int slices, int pitch, const float *bias, const int8_t *mask,
-                                  float *ctx, int ld_ctx, float alpha, int heads, int seq_length, int head_size,
-                                  void *stream);
-int cubert_attention_partials_f16(const float *partials, int slices, int pitch, const cubert_half *bias,
-                                  const int8_t *mask, cubert_half *ctx, int ld_ctx, float alpha, int heads,
-                                  int seq_length, int head_size, void *stream);
-
 /* Longest sequences first.  The long-sequence kernels (seq_length > 128) leave out key tiles (32 keys) whose mask
  * bytes are all zero, so a workgroup's time goes with its sequence's number of live tiles, and workgroups are handed
  * to the compute units in index order: a long sequence late in the batch starts late and the launch waits for it.
@@ -372,7 +357,7 @@ int cubert_gemm_skinny_packed_f16(void *handle, int M, int N, int K, float alpha
                                   int activation);
 
 /* The few-token product left as partial sums, for a consumer kernel that adds them while it loads its operand
- * (cubert_bias_res_ln_partials_*, cubert_attention_partials_*).  A few-token Dense kernel spends 2 of its 7-10 us
+ * (cubert_bias_res_ln_partials_*).  A few-token Dense kernel spends 2 of its 7-10 us
  * handing the K slices over to the workgroup that adds them; here every workgroup stores its slice and is done:
  *   partials[(slice * 32 + token) * pitch + feature] = sum over the slice's k of A[k, feature] * B[k, token]
  * for *slices slices, all 32 token rows (rows from N on are zero) and *pitch >= M features per row (fp32 whatever the

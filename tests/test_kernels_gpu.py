@@ -1014,58 +1014,6 @@ def test_bias_res_ln_from_partials_declines_what_it_cannot_do(K):
     assert K.bias_res_ln_partials(narrow, torch.zeros((4, 768), device="cuda"), v, v, v) is None  # rows narrower than hidden
 
 
-@pytest.mark.parametrize("name", ["f32", "f16"])
-@pytest.mark.parametrize("heads,masked", [(12, True), (12, False), (16, True), (2, True)])
-def test_attention_from_partials_has_the_bits_of_gemm_then_attention(K, name, heads, masked):
-    """One sequence of 32 tokens: Q|K|V projection left as K slices, attention core reading them."""
-    seq, d = 32, 64
-    hidden = heads * d
-    rng = np.random.default_rng(heads * 2 + masked)
-    blas = K.Blas()
-    W = dev(q(rng.normal(0, 0.05, hidden * 3 * hidden), name), tdt(name))          # [in, 3 * hidden]
-    X = dev(q(rng.normal(0, 1, seq * hidden), name), tdt(name))
-    bias = dev(q(rng.normal(0, 0.5, 3 * hidden), name), tdt(name))
-    mask = None
-    if masked:
-        m = np.ones(seq, np.int8)
-        m[rng.integers(5, seq):] = 0
-        m[2] = 0
-        mask = dev(m)
-    qkv = torch.zeros((seq, 3 * hidden), dtype=tdt(name), device="cuda")
-    assert blas.gemm_skinny(3 * hidden, seq, hidden, 1.0, W, 3 * hidden, X, hidden, qkv, 3 * hidden, bias=bias) is not None
-    want = K.attention_fused(qkv, mask, 1, heads, seq, d, 0.125)
-    assert want is not None
-    got = blas.gemm_skinny_partials(3 * hidden, seq, hidden, W, 3 * hidden, X, hidden)
-    assert got is not None
-    partials, slices, pitch = got
-    ctx = K.attention_partials(partials, bias, mask, heads, seq, d, 0.125)
-    assert ctx is not None
-    assert torch.equal(ctx, want)
-    # and against the oracle on the projection the GEMM stored
-    stored = host(qkv)
-    qh, kh, vh = (np.ascontiguousarray(x) for x in (stored[:, :hidden], stored[:, hidden:2 * hidden], stored[:, 2 * hidden:]))
-    scores = oracle.att_q_k(qh, kh, 1, seq, heads, d, alpha=0.125)
-    if name == "f16":
-        scores = oracle.round_to_half(scores)
-    if masked:
-        scores = scores + (-10000.0 * (1.0 - m.astype(np.float32)))[None, None, None, :]
-    p = oracle.softmax_(np.ascontiguousarray(scores.reshape(-1, seq), dtype=np.float32)).reshape(scores.shape)
-    if name == "f16":
-        p = oracle.round_to_half(p)
-    ref = oracle.att_qk_v(np.ascontiguousarray(p, dtype=np.float32), vh, 1, seq, heads, d).reshape(seq, hidden)
-    assert_close(host(ctx), ref, 2e-5 if name == "f32" else 2e-3, "attention from partials %s" % name)
-
-
-def test_attention_from_partials_declines_what_it_cannot_do(K):
-    partials = torch.zeros((3, 32, 2304), device="cuda")
-    bias = torch.zeros(2304, device="cuda")
-    assert K.attention_partials(partials, bias, None, 12, 16, 64, 0.125) is None     # not 32 tokens
-    assert K.attention_partials(partials, bias, None, 24, 32, 32, 0.125) is None     # head size 32
-    assert K.attention_partials(torch.zeros((3, 32, 2048), device="cuda"), bias, None, 12, 32, 64, 0.125) is None  # rows too narrow
-    many = torch.zeros((5, 32, 2304), device="cuda")
-    assert K.attention_partials(many, bias, None, 12, 32, 64, 0.125) is None         # more than four slices
-
-
 def test_gemm_skinny_declines_what_it_cannot_do(K):
     blas = K.Blas()
     x = torch.zeros(64 * 1024, device="cuda")
