@@ -51,8 +51,8 @@ TRAFFIC_PROFILE = "profiles/traffic_pmc.md"
 TRAFFIC_SOURCE = {  # kernel kind -> (source file under cubert_amd/csrc/kernels, first 16 hex digits of its SHA-256)
     "bias_gelu": ("elementwise.hip", "59dcc33f61344079"),
     "bias_tanh": ("elementwise.hip", "59dcc33f61344079"),
-    "bias_res_ln": ("layernorm.hip", "0adeeda2d66610ed"),
-    "embed_ln": ("layernorm.hip", "0adeeda2d66610ed"),
+    "bias_res_ln": ("layernorm.hip", "63cfef94a6b85850"),
+    "embed_ln": ("layernorm.hip", "63cfef94a6b85850"),
     "mask_scale_softmax": ("softmax.hip", "90a529eac55169fa"),
     "mean_pool": ("elementwise.hip", "59dcc33f61344079"),
     "classifier_head": ("elementwise.hip", "59dcc33f61344079"),
@@ -60,37 +60,37 @@ TRAFFIC_SOURCE = {  # kernel kind -> (source file under cubert_amd/csrc/kernels,
 }
 MEASURED_TRAFFIC = {
     "C1": {
-        "embed_ln": 25327911,
-        "attention_fused": 50081728,
-        "bias_res_ln": 37631154,
-        "bias_gelu": 100340722,
-        "classifier_head": 934418,
-        "mask_scale_softmax": 12589776
+        "embed_ln": 25327834,
+        "attention_fused": 50081947,
+        "bias_res_ln": 37631060,
+        "bias_gelu": 100340726,
+        "classifier_head": 934419,
+        "mask_scale_softmax": 12589780
     },
     "C2": {
-        "embed_ln": 12910635,
-        "attention_fused": 25138608,
-        "bias_res_ln": 18866021,
-        "bias_gelu": 50185067,
-        "mean_pool": 6325126,
+        "embed_ln": 12897102,
+        "attention_fused": 25138619,
+        "bias_res_ln": 18850804,
+        "bias_gelu": 50185082,
+        "mean_pool": 6325077,
         "classifier_head": 147249,
-        "mask_scale_softmax": 25117482
+        "mask_scale_softmax": 25117480
     },
     "C3": {
-        "embed_ln": 99735269,
-        "attention_fused": 128669160,
-        "bias_res_ln": 150207501,
-        "bias_gelu": 400907313,
+        "embed_ln": 99732176,
+        "attention_fused": 128669549,
+        "bias_res_ln": 150191566,
+        "bias_gelu": 400908911,
         "classifier_head": 308694,
-        "mask_scale_softmax": 801925725
+        "mask_scale_softmax": 801926098
     },
     "C4": {
-        "embed_ln": 133764546,
-        "attention_fused": 267267622,
-        "bias_res_ln": 200189416,
-        "bias_gelu": 534518936,
-        "classifier_head": 1199624,
-        "mask_scale_softmax": 267503672
+        "embed_ln": 133757147,
+        "attention_fused": 267267773,
+        "bias_res_ln": 200203032,
+        "bias_gelu": 534519157,
+        "classifier_head": 1199518,
+        "mask_scale_softmax": 267503966
     }
 }
 
