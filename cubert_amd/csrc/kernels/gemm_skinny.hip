@@ -17,8 +17,8 @@
 //
 // That hand-over (partial tile written through, ticket, partial tiles read back) is 2 us of a 7-10 us kernel.
 // gemm_skinny_partials leaves it out: every workgroup stores its partial tile and is done, and the kernel that
-// consumes the Dense layer's output (bias + residual + LayerNorm) adds the slices in the same slice order while it
-// loads its operand, which gives the same bits.
+// consumes the Dense layer's output (bias + residual + LayerNorm) adds the slices in slice order while it loads its
+// operand.
 
 #include <cstdio>
 #include <mutex>
@@ -243,8 +243,9 @@ int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, int packe
 // The same product left as partial tiles: partials[(slice * 32 + token) * pitch + feature] holds slice `slice` of
 // sum_k A[k, feature] B[k, token] for all 32 token rows (rows from N on are zero), *slices and *pitch say how many
 // and how wide.  No alpha, bias or activation: the consumer adds the slices in slice order (0.f + p0 + p1 + ...) and
-// goes on from there, which is what gemm_skinny's last workgroup does.  Same cut as gemm_skinny for the same
-// partial_floats; nothing is launched when the problem does not fit.
+// goes on from there, which is what gemm_skinny's last workgroup does.  The cut is gemm_skinny's, or a finer one
+// (below), so the sum agrees with gemm_skinny's result up to the order of the additions.  Nothing is launched when
+// the problem does not fit.
 template <typename T>
 int gemm_skinny_partials(int M, int N, int K, const T *A, int lda, int packed, const T *B, int ldb, float *partials,
                          size_t partial_floats, int *slices_out, int *pitch_out, hipStream_t stream) {
@@ -252,6 +253,22 @@ int gemm_skinny_partials(int M, int N, int K, const T *A, int lda, int packed, c
     SkinnyPlan plan;
     const int rc = gemm_skinny_plan<T>(M, N, K, A, lda, packed, B, ldb, M, 0, partial_floats, 0x7fffffff, &plan);
     if (rc) return rc;
+    // More slices cost this kernel nothing (it adds none of them), and a matrix with few feature blocks streams faster
+    // when more compute units pull on it: such a reduction is cut thinner than a pass of 16 chunks, up to about 192
+    // workgroups.  Measured at 768 x 768 (24 feature blocks) inside a forward pass: 3 slices of 16 chunks 7.2 us, 6 of 8
+    // and 8 of 6 6.5 us; 12 of 4 no better, and whoever adds the slices reads more of them.
+    constexpr int kThinTarget = 192;
+    if (plan.chunks_per_slice == kSkinnyWaves && plan.blocks * plan.slices < kThinTarget) {
+        const int chunks = K / kSkinnyChunk;
+        const int want = kThinTarget / plan.blocks;
+        int thin = (chunks + want - 1) / want;
+        const size_t tile = (size_t) 32 * plan.blocks * 32;  // floats per slice
+        while (thin < kSkinnyWaves && (size_t) ((chunks + thin - 1) / thin) * tile > partial_floats) ++thin;  // what fits
+        if (thin >= 1 && thin < kSkinnyWaves) {
+            plan.chunks_per_slice = thin;
+            plan.slices = (chunks + thin - 1) / thin;
+        }
+    }
     if ((size_t) plan.slices * 32 * plan.blocks * 32 > partial_floats) return CUBERT_UNSUPPORTED;
     const int chunks_per_slice = plan.chunks_per_slice;
     const dim3 grid(plan.blocks, plan.slices), block(kSkinnyThreads);
@@ -263,7 +280,7 @@ int gemm_skinny_partials(int M, int N, int K, const T *A, int lda, int packed, c
 #define CUBERT_SKINNY_PARTIALS(PACKED, PASSES)                                                                       \
     return launch(gemm_skinny_kernel<T, false, PACKED, PASSES>, grid, block, stream, A, lda, B, ldb, no_bias, no_output, \
                   M, M, N, K, 1.f, partials, no_counters, chunks_per_slice, 1)
-    if (chunks_per_slice == kSkinnyWaves) {
+    if (chunks_per_slice <= kSkinnyWaves) {
         if (packed) CUBERT_SKINNY_PARTIALS(true, 1);
         CUBERT_SKINNY_PARTIALS(false, 1);
     }

@@ -74,8 +74,9 @@ int cubert_bias_res_ln_f16(cubert_half *inout, const cubert_half *residual, cons
  *   a = storage type of (0.f + partials[(0 * 32 + r) * pitch + c] + partials[(1 * 32 + r) * pitch + c] + ...)
  *   x = a + bias + residual[r];  out[r] = beta + gamma * (x - mean) / sqrt(var + 1e-12)
  * i.e. cubert_gemm_skinny_* (alpha 1, no bias) followed by cubert_bias_res_ln_*, without the GEMM's hand-over between
- * workgroups: the same bits, except for 768 halves, where cubert_bias_res_ln_f16 runs a kernel that adds a row's sums
- * in another order (same inputs to the LayerNorm, last-bit differences after it).  `out` is written only (it may be any buffer but `residual`).  Shapes the
+ * workgroups.  Given the slices the result has the bits of cubert_bias_res_ln_* on their rounded sum, except for 768
+ * halves, where cubert_bias_res_ln_f16 runs a kernel that adds a row's sums in another order (same inputs to the
+ * LayerNorm, last-bit differences after it).  `out` is written only (it may be any buffer but `residual`).  Shapes the
  * register-resident LayerNorm kernels do not take (hidden not 64 * {2,4,8} * {1..5}) return CUBERT_UNSUPPORTED
  * and launch nothing.
  * replaces: Dense + layer_norm_<T> of BertOutput / the attention output for a request of at most 32 tokens,
@@ -362,8 +363,10 @@ int cubert_gemm_skinny_packed_f16(void *handle, int M, int N, int K, float alpha
  *   partials[(slice * 32 + token) * pitch + feature] = sum over the slice's k of A[k, feature] * B[k, token]
  * for *slices slices, all 32 token rows (rows from N on are zero) and *pitch >= M features per row (fp32 whatever the
  * storage type; no alpha, bias or activation).  Adding the slices in slice order, starting from 0.f, and rounding
- * to the storage type gives the bits cubert_gemm_skinny_* stores for alpha = 1 and no bias.  packed != 0: A is the
- * output of cubert_gemm_skinny_pack_* (lda ignored).  The cut is the one cubert_gemm_skinny_* makes; partials must
+ * to the storage type is what a consumer does; the result is cubert_gemm_skinny_*'s for alpha = 1 and no bias up to
+ * the order of the additions (the reduction may be cut into more slices here: nobody in this kernel has to add them,
+ * and a weight matrix with few feature blocks streams faster when more workgroups pull on it).  packed != 0: A is the
+ * output of cubert_gemm_skinny_pack_* (lda ignored).  partials must
  * hold partial_floats >= *slices * 32 * *pitch floats (1 << 20 is enough for every BERT-base/large Dense layer),
  * else CUBERT_UNSUPPORTED and nothing is launched; same conditions on K, B and ldb as cubert_gemm_skinny_*.
  * Asynchronous on the handle's stream.  No counterpart in the reference; same place as cubert_gemm_skinny_*
