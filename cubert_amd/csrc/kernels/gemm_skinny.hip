@@ -9,7 +9,8 @@
 //
 // Decomposition: a workgroup of 16 wavefronts owns 32 output features and a slice of K (256 values per
 // pass); each wavefront multiplies a [32 tokens x 16] block of B with a [16 x 32 features] block of A on
-// the matrix cores (v_mfma_f32_32x32x2_f32; fp16 storage is widened to fp32 in registers).  Every load of
+// the matrix cores (fp32: eight v_mfma_f32_32x32x2_f32; fp16: one v_mfma_f32_32x32x16_f16 on the operands as
+// they are stored, a sixteenth of the matrix-core time, fp32 accumulation either way).  Every load of
 // the wavefront is issued before the first MFMA.  The 16 partial tiles are summed through LDS in wavefront
 // order.  When K is cut into several slices (grid.y > 1) each workgroup stores its partial tile to a
 // workspace and the last workgroup to arrive for a feature block (ticket from an atomic counter) adds the
@@ -38,6 +39,21 @@ constexpr int kSkinnyChunk = 16;  // reduction values a wavefront consumes per p
 
 // Accumulator register i of the lane half hh holds this row of a 32x32 MFMA result (column = lane % 32).
 __device__ __forceinline__ int acc_row(int i, int hh) { return (i >> 2) * 8 + hh * 4 + (i & 3); }
+
+typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
+
+// acc[token, feature] += sum over the 16 reduction values of a chunk: lane (r, hh) brings the 8 values
+// k = hh * 8 + t of token r (x) and of feature r (w).
+__device__ __forceinline__ void chunk_mma(v16f32 &acc, const float (&x)[8], const float (&w)[8]) {
+#pragma unroll
+    for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[t], w[t], acc, 0, 0, 0);
+}
+__device__ __forceinline__ void chunk_mma(v16f32 &acc, const half_t (&x)[8], const half_t (&w)[8]) {
+    v8f16 a, b;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) a[t] = x[t], b[t] = w[t];
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+}
 
 // Weights in the order the kernel consumes them: for feature block fb and chunk c (16 reduction values), lane
 // (r, hh) finds its 8 operand values A[c*16 + hh*8 + t, fb*32 + r], t < 8, in 8 consecutive elements, so a
@@ -79,7 +95,8 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
         // consecutive values of one row of B (vector loads), the weight operand one column of 8 rows of A.
         // The loads of all PASSES chunks are issued before the first MFMA; a chunk past the slice is read
         // from the wavefront's first chunk (a valid address, no branch around the loads) with its tokens zeroed.
-        float x[PASSES][8], w[PASSES][8];
+        T x[PASSES][8], w[PASSES][8];
+        const T zero = from_f32<T>(0.f);
 #pragma unroll
         for (int p = 0; p < PASSES; ++p) {
             const int c = c0 + p * kSkinnyWaves;
@@ -90,7 +107,7 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
                 Vec<T, V> xv = Vec<T, V>{};
                 if (r < N) xv = load_vec<T, V>(B + (size_t) r * ldb + kb + u * V);
 #pragma unroll
-                for (int e = 0; e < V; ++e) x[p][u * V + e] = inside ? to_f32(xv.v[e]) : 0.f;
+                for (int e = 0; e < V; ++e) x[p][u * V + e] = inside ? xv.v[e] : zero;
             }
             if (PACKED) {
                 const T *src = A + (((size_t) blockIdx.x * chunks + (inside ? c : c0)) * kWave + lane) * 8;
@@ -98,20 +115,17 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
                 for (int u = 0; u < 8 / V; ++u) {
                     const Vec<T, V> wv = load_vec<T, V>(src + u * V);
 #pragma unroll
-                    for (int e = 0; e < V; ++e) w[p][u * V + e] = to_f32(wv.v[e]);
+                    for (int e = 0; e < V; ++e) w[p][u * V + e] = wv.v[e];
                 }
             } else {
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
-                    w[p][t] = feature < M ? to_f32(A[(size_t) (kb + t) * lda + feature]) : 0.f;
+                    w[p][t] = feature < M ? A[(size_t) (kb + t) * lda + feature] : zero;
                 }
             }
         }
 #pragma unroll
-        for (int p = 0; p < PASSES; ++p) {
-#pragma unroll
-            for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[p][t], w[p][t], acc, 0, 0, 0);
-        }
+        for (int p = 0; p < PASSES; ++p) chunk_mma(acc, x[p], w[p]);
     }
     // lane holds C[feature = m0 + r, token = acc_row(i, hh)]
 #pragma unroll
