@@ -42,17 +42,33 @@ __device__ __forceinline__ int acc_row(int i, int hh) { return (i >> 2) * 8 + hh
 
 typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
 
-// acc[token, feature] += sum over the 16 reduction values of a chunk: lane (r, hh) brings the 8 values
-// k = hh * 8 + t of token r (x) and of feature r (w).
-__device__ __forceinline__ void chunk_mma(v16f32 &acc, const float (&x)[8], const float (&w)[8]) {
+// The 8 reduction values k = hh * 8 + t a lane (r, hh) brings to a chunk, of token r or of feature r, in the form the
+// matrix instruction of the storage type takes them.
+template <typename T>
+struct ChunkOperand;
+template <>
+struct ChunkOperand<float> {
+    float v[8];
+    __device__ __forceinline__ void set(int t, float x) { v[t] = x; }
+    __device__ __forceinline__ void loaded() {}
+};
+template <>
+struct ChunkOperand<half_t> {
+    v8f16 v;
+    __device__ __forceinline__ void set(int t, half_t x) { v[t] = x; }
+    // Counts as a use: every operand has been requested before the first MFMA.  (One short instruction per chunk:
+    // nothing to gain from starting early, and left alone the compiler requests the last operand of a second pass
+    // only after the first pass's MFMA, a second memory latency.)
+    __device__ __forceinline__ void loaded() { asm volatile("" : "+v"(v)); }
+};
+
+// acc[token, feature] += sum over the 16 reduction values of a chunk
+__device__ __forceinline__ void chunk_mma(v16f32 &acc, const ChunkOperand<float> &x, const ChunkOperand<float> &w) {
 #pragma unroll
-    for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[t], w[t], acc, 0, 0, 0);
+    for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.v[t], w.v[t], acc, 0, 0, 0);
 }
-__device__ __forceinline__ void chunk_mma(v16f32 &acc, const half_t (&x)[8], const half_t (&w)[8]) {
-    v8f16 a, b;
-#pragma unroll
-    for (int t = 0; t < 8; ++t) a[t] = x[t], b[t] = w[t];
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+__device__ __forceinline__ void chunk_mma(v16f32 &acc, const ChunkOperand<half_t> &x, const ChunkOperand<half_t> &w) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(x.v, w.v, acc, 0, 0, 0);
 }
 
 // Weights in the order the kernel consumes them: for feature block fb and chunk c (16 reduction values), lane
@@ -95,19 +111,20 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
         // consecutive values of one row of B (vector loads), the weight operand one column of 8 rows of A.
         // The loads of all PASSES chunks are issued before the first MFMA; a chunk past the slice is read
         // from the wavefront's first chunk (a valid address, no branch around the loads) with its tokens zeroed.
-        T x[PASSES][8], w[PASSES][8];
+        ChunkOperand<T> x[PASSES], w[PASSES];
         const T zero = from_f32<T>(0.f);
 #pragma unroll
         for (int p = 0; p < PASSES; ++p) {
             const int c = c0 + p * kSkinnyWaves;
             const bool inside = c < c_end;
             const int kb = (inside ? c : c0) * kSkinnyChunk + hh * 8;
+            // (token rows from N on read row N - 1 and count as zero, weight columns from M on read column M - 1 and
+            // are never stored: no load stands under a branch, so the first pass can start while the second is on its way)
 #pragma unroll
             for (int u = 0; u < 8 / V; ++u) {
-                Vec<T, V> xv = Vec<T, V>{};
-                if (r < N) xv = load_vec<T, V>(B + (size_t) r * ldb + kb + u * V);
+                const Vec<T, V> xv = load_vec<T, V>(B + (size_t) (r < N ? r : N - 1) * ldb + kb + u * V);
 #pragma unroll
-                for (int e = 0; e < V; ++e) x[p][u * V + e] = inside ? xv.v[e] : zero;
+                for (int e = 0; e < V; ++e) x[p].set(u * V + e, inside && r < N ? xv.v[e] : zero);
             }
             if (PACKED) {
                 const T *src = A + (((size_t) blockIdx.x * chunks + (inside ? c : c0)) * kWave + lane) * 8;
@@ -115,15 +132,20 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
                 for (int u = 0; u < 8 / V; ++u) {
                     const Vec<T, V> wv = load_vec<T, V>(src + u * V);
 #pragma unroll
-                    for (int e = 0; e < V; ++e) w[p][u * V + e] = wv.v[e];
+                    for (int e = 0; e < V; ++e) w[p].set(u * V + e, wv.v[e]);
                 }
             } else {
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
-                    w[p][t] = feature < M ? A[(size_t) (kb + t) * lda + feature] : zero;
+                    w[p].set(t, A[(size_t) (kb + t) * lda + (feature < M ? feature : M - 1)]);
                 }
             }
         }
+        // nothing moves across this line: every load of the wavefront is requested before its first MFMA (the waits
+        // are placed per operand afterwards, so a first pass still starts while the second is on its way)
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) x[p].loaded(), w[p].loaded();
 #pragma unroll
         for (int p = 0; p < PASSES; ++p) chunk_mma(acc, x[p], w[p]);
     }
