@@ -39,7 +39,7 @@ Transformer<T>::Transformer(void *cublas, const std::string &var_prefix,
     const size_t H = hidden_size, I = intermediate_size;
     // The re-ordered copies pay off for 2-byte weights (the plain layout makes the few-token kernel read 64-byte
     // pieces): measured 2 us per GEMM at hidden 768; for 4-byte weights the gain is within 5 %, not worth the memory.
-    keep_packed = sizeof(T) == 2 && seq_length <= 32 && H % 16 == 0 && I % 16 == 0;
+    keep_packed = sizeof(T) == 2 && seq_length <= 64 && H % 16 == 0 && I % 16 == 0;
     // The library's fp16 GEMMs are 10-19 % faster with both operands contiguous along the reduction (measured at
     // 32768 tokens on every Dense shape of BERT-base and BERT-large, same bits out); its fp32 GEMMs do not care.
     // Half-precision models therefore keep their Dense kernels [out, in], transposed once here.
@@ -195,7 +195,7 @@ void Transformer<T>::layout_buffers() {
     layer_output[0] = buffers.take<T>(M * H);
     layer_output[1] = buffers.take<T>(M * H);
     if (split_dense) split_operand = buffers.take<half>(M * 3 * (H > intermediate_size ? H : intermediate_size));
-    if (seq_length <= 32) few_token_partials = buffers.take<float>(kFewTokenPartialFloats);
+    if (seq_length <= 64) few_token_partials = buffers.take<float>(kFewTokenPartialFloats);
 }
 
 template <typename T>
@@ -302,7 +302,7 @@ bool Transformer<T>::dense(int out_features, int tokens, int in_features, const 
     Timed t(profiler, profiler != nullptr ? profiler->dense_kind(kind) : Profiler::kDenseGemm, stream);
     if (ld_out == 0) ld_out = out_features;
     // (the few-token kernel reads [in, out] kernels or its own copy of them, not transposed ones)
-    if (tokens <= 32 && (packed != nullptr || (!transposed_kernels && gelu && dense_gelu_fits))) {
+    if (tokens <= few_token_limit(kind) && (packed != nullptr || (!transposed_kernels && (gelu || tokens > 32) && dense_gelu_fits))) {
         const bool with_bias = bias_in_gemm || gelu;
         if (cuBERT::dense_few_tokens(cublas, out_features, tokens, in_features, kernel, out_features, packed, in,
                                      in_features, out, ld_out, with_bias ? bias : nullptr, gelu)) {
@@ -337,6 +337,22 @@ void Transformer<T>::dense_split(int out_features, int tokens, int in_features, 
     }
 }
 
+// Up to how many tokens a Dense layer runs on the few-token kernel.  32 for all of them; 64 where the kernel with two
+// blocks of 32 tokens per wavefront is ahead of the library.  Measured at BERT-base, batch 2 x seq 32, a launch
+// event-timed inside the forward pass, library against kernel -- fp32: attention output 9.1 / 7.6 us, output
+// 20.4 / 15.1 us, but Q|K|V 11.7 / 12.5 and intermediate + GELU 16.4 / 18.7 (the fp32 MFMAs of a second token block
+// cost what the library's tiles do not); fp16: attention output 8.6 / 6.5, intermediate + GELU 14.6 / 10.7, output
+// 10.4 / 7.7, Q|K|V 8.5 / 10.1.  Forward pass 0.665 -> 0.61 ms (fp32), 0.541 -> 0.423 ms (fp16).
+template <typename T>
+int Transformer<T>::few_token_limit(Profiler::Kind kind) const {
+    switch (kind) {
+        case Profiler::kDenseAttentionOutput:
+        case Profiler::kDenseOutput: return 64;
+        case Profiler::kDenseIntermediate: return sizeof(T) == 2 ? 64 : 32;
+        default: return 32;
+    }
+}
+
 // CUBERT_FEW_TOKEN_SLICES=0 in the environment keeps the few-token Dense kernels adding their own K slices.
 static bool few_token_slices_enabled() {
     static const bool on = [] {
@@ -351,7 +367,7 @@ void Transformer<T>::dense_norm(int tokens, int in_features, const T *kernel, co
                                 const T *residual, const T *beta, const T *gamma, T *out, Profiler::Kind kind) {
     void *stream = cuBERT::blas_get_stream(cublas);
     const int H = (int) hidden_size;
-    if (tokens <= 32 && slices_to_norm && few_token_partials != nullptr && few_token_slices_enabled() &&
+    if (tokens <= few_token_limit(kind) && slices_to_norm && few_token_partials != nullptr && few_token_slices_enabled() &&
         (packed != nullptr || !transposed_kernels)) {
         int slices = 0, pitch = 0;
         bool done = false;

@@ -4,7 +4,8 @@
 // with device pointers, returning a device pointer to [batch, seq, hidden].
 //
 // Inside, a layer is 8 launches (7 for at most 32 tokens, where the two Dense kernels in front of a LayerNorm also
-// leave their K slices to it instead of adding them up themselves):
+// leave their K slices to it instead of adding them up themselves; up to 64 tokens those two, and in half precision
+// the intermediate one, still run on the few-token kernel):
 //   qkv   = x * [Wq|Wk|Wv] + [bq|bk|bv]          one GEMM, bias in its epilogue
 //   ctx   = softmax((1/sqrt d) Q K^T + mask) V    one attention kernel (scores stay in registers); where its
 //                                                 shape limits do not hold: scores kernel or batched GEMM into
@@ -118,6 +119,9 @@ private:
     void dense_norm(int tokens, int in_features, const T *kernel, const T *packed, const T *in, const T *bias,
                     const T *residual, const T *beta, const T *gamma, T *out, Profiler::Kind kind);
 
+    // up to how many tokens the Dense layer of this kind runs on the few-token kernel (32 or 64)
+    int few_token_limit(Profiler::Kind kind) const;
+
     void *cublas;
     Profiler *profiler = nullptr;
     bool slices_to_norm = true;        // few-token Dense layers hand their K slices to the LayerNorm (cleared when declined)
@@ -147,7 +151,7 @@ private:
     T *layer_output[2];      // [M, hidden], alternating between layers
     half *split_operand = nullptr;  // [M, 3 * max(hidden, intermediate)] two-term rows of the current Dense input
     static constexpr size_t kFewTokenPartialFloats = (size_t) 1 << 20;
-    float *few_token_partials = nullptr;  // K slices of the current few-token Dense layer (seq_length <= 32 only)
+    float *few_token_partials = nullptr;  // K slices of the current few-token Dense layer (seq_length <= 64 only)
 };
 
 }  // namespace cuBERT

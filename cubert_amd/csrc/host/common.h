@@ -82,7 +82,7 @@ inline void blas_gemm(void *handle, bool TransA, bool TransB, int M, int N, int 
                       const half *B, int ldb, float beta, half *C, int ldc, const half *bias = nullptr) {
     CUBERT_CHECK(cubert_gemm_f16(handle, TransA, TransB, M, N, K, alpha, h(A), lda, h(B), ldb, beta, h(C), ldc, h(bias)));
 }
-// A Dense layer for at most 32 tokens on the few-token kernel (column-major C[M, N] = [gelu](A B + bias), N <= 32),
+// A Dense layer for at most 64 tokens on the few-token kernel (column-major C[M, N] = [gelu](A B + bias), N <= 64),
 // on the weights in its own order when `packed` is given; false when the kernel does not take the problem
 // (the caller then runs blas_gemm).  No counterpart in the reference.
 inline bool dense_few_tokens(void *handle, int M, int N, int K, const float *A, int lda, const float *packed,
@@ -103,7 +103,8 @@ inline bool dense_few_tokens(void *handle, int M, int N, int K, const half *A, i
     return true;
 }
 // The same product left as K slices for the kernel that consumes it (layer_norm_partials):
-// partials[(slice * 32 + token) * pitch + feature], fp32; false when the kernel does not take the problem.
+// partials[(slice * R + token) * pitch + feature], fp32, R = N rounded up to 32; false when the kernel does not take
+// the problem.
 inline bool dense_few_tokens_partials(void *handle, int M, int N, int K, const float *A, int lda, const float *packed,
                                       const float *B, int ldb, float *partials, size_t partial_floats, int *slices,
                                       int *pitch) {
@@ -122,7 +123,7 @@ inline bool dense_few_tokens_partials(void *handle, int M, int N, int K, const h
     CUBERT_CHECK(rc);
     return true;
 }
-// out = LayerNorm(storage type of (sum of the slices) + bias + residual) for at most 32 rows; false when declined
+// out = LayerNorm(storage type of (sum of the slices) + bias + residual) for at most 64 rows; false when declined
 inline bool layer_norm_partials(float *out, const float *partials, int slices, int pitch, const float *residual,
                                 const float *bias, const float *beta, const float *gamma, int rows, int hidden,
                                 void *stream) {

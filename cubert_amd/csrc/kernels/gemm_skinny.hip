@@ -1,5 +1,5 @@
 // Dense layer for a handful of tokens:  C[M, N] = alpha * A[M, K] * B[K, N] + bias  (column-major, no
-// transposes) with N <= 32.  In the row-major picture of a Dense layer A is the weight matrix [in, out]
+// transposes) with N <= 64.  In the row-major picture of a Dense layer A is the weight matrix [in, out]
 // (M = out features, K = in features), B the activations of N tokens and C their outputs.
 //
 // With so few tokens the GEMM is a single pass over the weights: every weight is used once per token and
@@ -36,6 +36,7 @@ typedef float v16f32 __attribute__((ext_vector_type(16)));
 constexpr int kSkinnyWaves = 16;
 constexpr int kSkinnyThreads = kSkinnyWaves * kWave;
 constexpr int kSkinnyChunk = 16;  // reduction values a wavefront consumes per pass: 8 per lane half
+constexpr int kSkinnyMaxTokens = 64;  // two blocks of 32 tokens per wavefront
 
 // Accumulator register i of the lane half hh holds this row of a 32x32 MFMA result (column = lane % 32).
 __device__ __forceinline__ int acc_row(int i, int hh) { return (i >> 2) * 8 + hh * 4 + (i & 3); }
@@ -88,7 +89,7 @@ __global__ __launch_bounds__(kBlock) void gemm_skinny_pack_kernel(const T *__res
     packed[idx] = feature < M ? A[(size_t) k * lda + feature] : from_f32<T>(0.f);
 }
 
-template <typename T, bool GELU, bool PACKED, int PASSES>
+template <typename T, bool GELU, bool PACKED, int PASSES, int TB>
 __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__restrict__ A, int lda,
                                                                      const T *__restrict__ B, int ldb,
                                                                      const T *__restrict__ bias, T *__restrict__ C,
@@ -105,13 +106,16 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
     const int c_begin = blockIdx.y * chunks_per_slice;
     const int c_end = c_begin + chunks_per_slice < chunks ? c_begin + chunks_per_slice : chunks;
 
-    v16f32 acc = v16f32{};
+    // TB blocks of 32 tokens: a wavefront multiplies its weights with each of them (the weights are loaded once)
+    v16f32 acc[TB];
+#pragma unroll
+    for (int tb = 0; tb < TB; ++tb) acc[tb] = v16f32{};
     for (int c0 = c_begin + wave; c0 < c_end; c0 += kSkinnyWaves * PASSES) {
         // reduction slot of MFMA t in lane half hh is k = c*16 + hh*8 + t: the token operand of a lane is 8
         // consecutive values of one row of B (vector loads), the weight operand one column of 8 rows of A.
         // The loads of all PASSES chunks are issued before the first MFMA; a chunk past the slice is read
         // from the wavefront's first chunk (a valid address, no branch around the loads) with its tokens zeroed.
-        ChunkOperand<T> x[PASSES], w[PASSES];
+        ChunkOperand<T> x[PASSES][TB], w[PASSES];
         const T zero = from_f32<T>(0.f);
 #pragma unroll
         for (int p = 0; p < PASSES; ++p) {
@@ -121,10 +125,14 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
             // (token rows from N on read row N - 1 and count as zero, weight columns from M on read column M - 1 and
             // are never stored: no load stands under a branch, so the first pass can start while the second is on its way)
 #pragma unroll
-            for (int u = 0; u < 8 / V; ++u) {
-                const Vec<T, V> xv = load_vec<T, V>(B + (size_t) (r < N ? r : N - 1) * ldb + kb + u * V);
+            for (int tb = 0; tb < TB; ++tb) {
+                const int row = tb * 32 + r;
 #pragma unroll
-                for (int e = 0; e < V; ++e) x[p].set(u * V + e, inside && r < N ? xv.v[e] : zero);
+                for (int u = 0; u < 8 / V; ++u) {
+                    const Vec<T, V> xv = load_vec<T, V>(B + (size_t) (row < N ? row : N - 1) * ldb + kb + u * V);
+#pragma unroll
+                    for (int e = 0; e < V; ++e) x[p][tb].set(u * V + e, inside && row < N ? xv.v[e] : zero);
+                }
             }
             if (PACKED) {
                 const T *src = A + (((size_t) blockIdx.x * chunks + (inside ? c : c0)) * kWave + lane) * 8;
@@ -145,23 +153,37 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
         // are placed per operand afterwards, so a first pass still starts while the second is on its way)
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int p = 0; p < PASSES; ++p) x[p].loaded(), w[p].loaded();
+        for (int p = 0; p < PASSES; ++p) {
+            w[p].loaded();
 #pragma unroll
-        for (int p = 0; p < PASSES; ++p) chunk_mma(acc, x[p], w[p]);
+            for (int tb = 0; tb < TB; ++tb) x[p][tb].loaded();
+        }
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) {
+#pragma unroll
+            for (int tb = 0; tb < TB; ++tb) chunk_mma(acc[tb], x[p][tb], w[p]);
+        }
     }
-    // lane holds C[feature = m0 + r, token = acc_row(i, hh)]
+    // lane holds C[feature = m0 + r, token = tb * 32 + acc_row(i, hh)]; one output element per thread and token block
+    const int token = threadIdx.x >> 5, f = threadIdx.x & 31;
+    float sum[TB];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) red[wave][acc_row(i, hh) * 32 + r] = acc[i];
-    __syncthreads();
-
-    const int token = threadIdx.x >> 5, f = threadIdx.x & 31;  // one output element per thread
-    float sum = 0.f;
+    for (int tb = 0; tb < TB; ++tb) {
+        if (tb > 0) __syncthreads();  // the sums of the block before have been read
 #pragma unroll
-    for (int w = 0; w < kSkinnyWaves; ++w) sum += red[w][threadIdx.x];
-    const bool live = token < N && m0 + f < M;
+        for (int i = 0; i < 16; ++i) red[wave][acc_row(i, hh) * 32 + r] = acc[tb][i];
+        __syncthreads();
+        sum[tb] = 0.f;
+#pragma unroll
+        for (int w = 0; w < kSkinnyWaves; ++w) sum[tb] += red[w][threadIdx.x];
+    }
     const int slices = gridDim.y;
-    if (leave_partials) {  // (uniform) the consumer adds the slices: partials[slice][token][feature], all 32 token rows
-        partials[((size_t) blockIdx.y * 32 + token) * ((size_t) gridDim.x * 32) + m0 + f] = sum;
+    const size_t pitch = (size_t) gridDim.x * 32;  // features, padded to whole blocks
+    if (leave_partials) {  // (uniform) the consumer adds the slices: partials[slice][token][feature], all TB * 32 rows
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb) {
+            partials[((size_t) (blockIdx.y * TB + tb) * 32 + token) * pitch + m0 + f] = sum[tb];
+        }
         return;
     }
     if (slices > 1) {
@@ -169,9 +191,11 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
         // write back / invalidate a whole L2 per call.  Instead every access that crosses workgroups is a
         // relaxed device-scope atomic: such stores write through, such loads read past the die-local cache,
         // and a store has reached the coherent level once the wavefront's store counter has drained.
-        const size_t pitch = (size_t) gridDim.x * 32;  // features, padded to whole blocks
-        __hip_atomic_store(&partials[((size_t) blockIdx.y * 32 + token) * pitch + m0 + f], sum, __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb) {
+            __hip_atomic_store(&partials[((size_t) (blockIdx.y * TB + tb) * 32 + token) * pitch + m0 + f], sum[tb],
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's partial sums are written
         __syncthreads();                     // ... and so are the other wavefronts' (and red[] is free)
         int *ticket = reinterpret_cast<int *>(&red[0][0]);
@@ -181,27 +205,35 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
         __syncthreads();
         if (*ticket != slices - 1) return;
         // last workgroup of this feature block: every slice's partial tile is complete
-        sum = 0.f;
-        for (int s0 = 0; s0 < slices; s0 += 16) {  // up to 16 loads in flight, added in slice order
-            float p[16];
 #pragma unroll
-            for (int u = 0; u < 16; ++u) {
-                p[u] = s0 + u < slices ? __hip_atomic_load(&partials[((size_t) (s0 + u) * 32 + token) * pitch + m0 + f],
-                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                                       : 0.f;
+        for (int tb = 0; tb < TB; ++tb) {
+            sum[tb] = 0.f;
+            for (int s0 = 0; s0 < slices; s0 += 16) {  // up to 16 loads in flight, added in slice order
+                float p[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    p[u] = s0 + u < slices
+                               ? __hip_atomic_load(&partials[((size_t) ((s0 + u) * TB + tb) * 32 + token) * pitch + m0 + f],
+                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                               : 0.f;
+                }
+#pragma unroll
+                for (int u = 0; u < 16; ++u) sum[tb] += p[u];
             }
-#pragma unroll
-            for (int u = 0; u < 16; ++u) sum += p[u];
         }
         if (threadIdx.x == 0) {  // ready for the next launch
             __hip_atomic_store(&counters[blockIdx.x], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
-    if (live) {
-        float v = alpha * sum;
-        if (bias != nullptr) v += to_f32(bias[m0 + f]);
-        if (GELU) v = GeluOp<T>()(v);
-        C[(size_t) token * ldc + m0 + f] = from_f32<T>(v);
+    if (m0 + f < M) {
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb) {
+            if (tb * 32 + token >= N) break;
+            float v = alpha * sum[tb];
+            if (bias != nullptr) v += to_f32(bias[m0 + f]);
+            if (GELU) v = GeluOp<T>()(v);
+            C[(size_t) (tb * 32 + token) * ldc + m0 + f] = from_f32<T>(v);
+        }
     }
 }
 
@@ -209,7 +241,7 @@ __global__ __launch_bounds__(kSkinnyThreads) void gemm_skinny_kernel(const T *__
 
 // How a problem is cut: feature blocks, K slices and the chunks of 16 reduction values per slice.
 struct SkinnyPlan {
-    int blocks = 0, slices = 0, chunks_per_slice = 0;
+    int blocks = 0, slices = 0, chunks_per_slice = 0, token_blocks = 0;
 };
 
 // Every check gemm_skinny makes and the cut it would launch with; launches nothing.  Returns 0, CUBERT_BAD_ARGUMENT or
@@ -218,12 +250,13 @@ template <typename T>
 int gemm_skinny_plan(int M, int N, int K, const T *A, int lda, int packed, const T *B, int ldb, int ldc, int activation,
                      size_t partial_floats, int n_counters, SkinnyPlan *plan) {
     if (activation != 0 && activation != 1) return CUBERT_BAD_ARGUMENT;
-    if (M <= 0 || N <= 0 || N > 32 || K <= 0 || K % kSkinnyChunk != 0) return CUBERT_UNSUPPORTED;
+    if (M <= 0 || N <= 0 || N > kSkinnyMaxTokens || K <= 0 || K % kSkinnyChunk != 0) return CUBERT_UNSUPPORTED;
     if ((!packed && lda < M) || ldb < K || ldc < M) return CUBERT_BAD_ARGUMENT;
     if (packed && !is_aligned(A, 16)) return CUBERT_BAD_ARGUMENT;
     if (!is_aligned(B, 16) || (ldb * sizeof(T)) % 16 != 0) return CUBERT_UNSUPPORTED;
     const int blocks = (M + 31) / 32;
     const int chunks = K / kSkinnyChunk;
+    const int token_blocks = (N + 31) / 32;
     // One pass (16 reduction values) per wavefront, unless that makes more workgroups than the chip has compute
     // units: a second round of workgroups costs more than a second pass of every wavefront (measured at
     // 768 x 3072 and 3072 x 768: 10.3 -> 9.5 us), while fewer, longer workgroups lose where one round is enough
@@ -232,16 +265,20 @@ int gemm_skinny_plan(int M, int N, int K, const T *A, int lda, int packed, const
     constexpr int kComputeUnits = 256;
     int chunks_per_slice = kSkinnyWaves;
     int slices = (chunks + chunks_per_slice - 1) / chunks_per_slice;
-    if (slices > 1 && (long long) slices * blocks > kComputeUnits && (packed || sizeof(T) == 4)) {
+    // With two token blocks of 4-byte operands the matrix-core time per pass doubles and outweighs both (768 x 3072 at
+    // 64 tokens: two passes 17.0 us, one 15.1 us; 2-byte operands, whose MFMAs are short, keep two: 8.0 against 8.7 us).
+    if (slices > 1 && (long long) slices * blocks > kComputeUnits && (packed || sizeof(T) == 4) &&
+        !(sizeof(T) == 4 && token_blocks > 1)) {
         chunks_per_slice = 2 * kSkinnyWaves;
         slices = (chunks + chunks_per_slice - 1) / chunks_per_slice;
     }
-    while (slices > 1 && (size_t) slices * 32 * blocks * 32 > partial_floats) {
+    while (slices > 1 && (size_t) slices * token_blocks * 32 * blocks * 32 > partial_floats) {
         chunks_per_slice += kSkinnyWaves;
         slices = (chunks + chunks_per_slice - 1) / chunks_per_slice;
     }
     if (blocks > 65535 || slices > 65535 || (slices > 1 && blocks > n_counters)) return CUBERT_UNSUPPORTED;
     plan->blocks = blocks, plan->slices = slices, plan->chunks_per_slice = chunks_per_slice;
+    plan->token_blocks = token_blocks;
     return 0;
 }
 
@@ -258,14 +295,17 @@ int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, int packe
     if (rc) return rc;
     const int blocks = plan.blocks, slices = plan.slices, chunks_per_slice = plan.chunks_per_slice;
     const dim3 grid(blocks, slices), block(kSkinnyThreads);
+#define CUBERT_SKINNY_LAUNCH_TB(GELU, PACKED, PASSES, TB)                                                            \
+    return launch(gemm_skinny_kernel<T, GELU, PACKED, PASSES, TB>, grid, block, stream, A, lda, B, ldb, bias, C, ldc, M, \
+                  N, K, alpha, partials, counters, chunks_per_slice, 0)
 #define CUBERT_SKINNY_LAUNCH(GELU, PACKED)                                                                           \
     do {                                                                                                             \
-        if (chunks_per_slice == kSkinnyWaves) {                                                                      \
-            return launch(gemm_skinny_kernel<T, GELU, PACKED, 1>, grid, block, stream, A, lda, B, ldb, bias, C, ldc, M, \
-                          N, K, alpha, partials, counters, chunks_per_slice, 0);                                     \
+        if (plan.token_blocks == 1) {                                                                                \
+            if (chunks_per_slice == kSkinnyWaves) CUBERT_SKINNY_LAUNCH_TB(GELU, PACKED, 1, 1);                       \
+            CUBERT_SKINNY_LAUNCH_TB(GELU, PACKED, 2, 1);                                                             \
         }                                                                                                            \
-        return launch(gemm_skinny_kernel<T, GELU, PACKED, 2>, grid, block, stream, A, lda, B, ldb, bias, C, ldc, M, N, \
-                      K, alpha, partials, counters, chunks_per_slice, 0);                                            \
+        if (chunks_per_slice == kSkinnyWaves) CUBERT_SKINNY_LAUNCH_TB(GELU, PACKED, 1, 2);                           \
+        CUBERT_SKINNY_LAUNCH_TB(GELU, PACKED, 2, 2);                                                                 \
     } while (0)
     if (activation == 1) {
         if (packed) CUBERT_SKINNY_LAUNCH(true, true);
@@ -273,6 +313,7 @@ int gemm_skinny(int M, int N, int K, float alpha, const T *A, int lda, int packe
     }
     if (packed) CUBERT_SKINNY_LAUNCH(false, true);
     CUBERT_SKINNY_LAUNCH(false, false);
+#undef CUBERT_SKINNY_LAUNCH_TB
 #undef CUBERT_SKINNY_LAUNCH
 }
 
@@ -298,14 +339,14 @@ int gemm_skinny_partials(int M, int N, int K, const T *A, int lda, int packed, c
         const int chunks = K / kSkinnyChunk;
         const int want = kThinTarget / plan.blocks;
         int thin = (chunks + want - 1) / want;
-        const size_t tile = (size_t) 32 * plan.blocks * 32;  // floats per slice
+        const size_t tile = (size_t) plan.token_blocks * 32 * plan.blocks * 32;  // floats per slice
         while (thin < kSkinnyWaves && (size_t) ((chunks + thin - 1) / thin) * tile > partial_floats) ++thin;  // what fits
         if (thin >= 1 && thin < kSkinnyWaves) {
             plan.chunks_per_slice = thin;
             plan.slices = (chunks + thin - 1) / thin;
         }
     }
-    if ((size_t) plan.slices * 32 * plan.blocks * 32 > partial_floats) return CUBERT_UNSUPPORTED;
+    if ((size_t) plan.slices * plan.token_blocks * 32 * plan.blocks * 32 > partial_floats) return CUBERT_UNSUPPORTED;
     const int chunks_per_slice = plan.chunks_per_slice;
     const dim3 grid(plan.blocks, plan.slices), block(kSkinnyThreads);
     *slices_out = plan.slices;
@@ -313,15 +354,21 @@ int gemm_skinny_partials(int M, int N, int K, const T *A, int lda, int packed, c
     const T *no_bias = nullptr;
     T *no_output = nullptr;
     int *no_counters = nullptr;
-#define CUBERT_SKINNY_PARTIALS(PACKED, PASSES)                                                                       \
-    return launch(gemm_skinny_kernel<T, false, PACKED, PASSES>, grid, block, stream, A, lda, B, ldb, no_bias, no_output, \
-                  M, M, N, K, 1.f, partials, no_counters, chunks_per_slice, 1)
-    if (chunks_per_slice <= kSkinnyWaves) {
-        if (packed) CUBERT_SKINNY_PARTIALS(true, 1);
-        CUBERT_SKINNY_PARTIALS(false, 1);
-    }
-    if (packed) CUBERT_SKINNY_PARTIALS(true, 2);
-    CUBERT_SKINNY_PARTIALS(false, 2);
+#define CUBERT_SKINNY_PARTIALS(PACKED, PASSES, TB)                                                                   \
+    return launch(gemm_skinny_kernel<T, false, PACKED, PASSES, TB>, grid, block, stream, A, lda, B, ldb, no_bias,    \
+                  no_output, M, M, N, K, 1.f, partials, no_counters, chunks_per_slice, 1)
+#define CUBERT_SKINNY_PARTIALS_TB(TB)                                                                                \
+    do {                                                                                                             \
+        if (chunks_per_slice <= kSkinnyWaves) {                                                                      \
+            if (packed) CUBERT_SKINNY_PARTIALS(true, 1, TB);                                                         \
+            CUBERT_SKINNY_PARTIALS(false, 1, TB);                                                                    \
+        }                                                                                                            \
+        if (packed) CUBERT_SKINNY_PARTIALS(true, 2, TB);                                                             \
+        CUBERT_SKINNY_PARTIALS(false, 2, TB);                                                                        \
+    } while (0)
+    if (plan.token_blocks == 1) CUBERT_SKINNY_PARTIALS_TB(1);
+    CUBERT_SKINNY_PARTIALS_TB(2);
+#undef CUBERT_SKINNY_PARTIALS_TB
 #undef CUBERT_SKINNY_PARTIALS
 }
 

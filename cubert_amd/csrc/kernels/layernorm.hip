@@ -146,9 +146,10 @@ __device__ __forceinline__ void load_floats(const float *__restrict__ p, float (
 }
 
 // bias + residual + LayerNorm of a Dense layer that the few-token GEMM left as K slices
-// (partials[(slice * 32 + row) * pitch + col], fp32): the slices are added here, in slice order from 0.f, and the
+// (partials[(slice * R + row) * pitch + col], fp32, R = rows rounded up to 32): the slices are added here, in slice
+// order from 0.f, and the
 // sum is rounded to the storage type before anything else happens to it -- the value the GEMM's own last workgroup
-// would have stored -- so the result has the bits of GEMM followed by bias_res_ln.  At most 32 rows.
+// would have stored -- so the result has the bits of GEMM followed by bias_res_ln.  At most 64 rows.
 template <typename T, int VEC, int CHUNKS, bool HAS_BIAS>
 __global__ __launch_bounds__(kBlock) void bias_res_ln_partials_kernel(T *__restrict__ out,
                                                                       const float *__restrict__ partials, int slices,
@@ -162,7 +163,7 @@ __global__ __launch_bounds__(kBlock) void bias_res_ln_partials_kernel(T *__restr
     if (row >= rows) return;
     const int lane = threadIdx.x & (kWave - 1);
     const float *prow = partials + (size_t) row * pitch;
-    const size_t slice_stride = (size_t) 32 * pitch;
+    const size_t slice_stride = (size_t) ((rows + 31) / 32 * 32) * pitch;  // whole blocks of 32 token rows per slice
     const T *res = residual + (size_t) row * H;
 
     Vec<T, VEC> r[CHUNKS], bi[CHUNKS], g[CHUNKS], be[CHUNKS];
@@ -494,7 +495,7 @@ int bias_res_ln_partials(T *out, const float *partials, int slices, int pitch, c
     if (rows < 0 || hidden <= 0 || slices <= 0 || !out || !partials || !residual || !beta || !gamma) {
         return CUBERT_BAD_ARGUMENT;
     }
-    if (rows > 32 || pitch < hidden || pitch % 4 != 0 || !is_aligned(partials, 16)) return CUBERT_UNSUPPORTED;
+    if (rows > 64 || pitch < hidden || pitch % 4 != 0 || !is_aligned(partials, 16)) return CUBERT_UNSUPPORTED;
     if (rows == 0) return 0;
     hipStream_t s = (hipStream_t) stream;
     // a wavefront per workgroup: what a row waits for is its slices arriving, and a compute unit pulls them at a

@@ -277,7 +277,7 @@ class Blas(object):
         return C
 
     def gemm_skinny(self, M, N, K, alpha, A, lda, B, ldb, C, ldc, bias=None, gelu=False):
-        """C = [gelu](alpha A B (+ bias)) with the few-token kernel (N <= 32); None when the problem does not fit."""
+        """C = [gelu](alpha A B (+ bias)) with the few-token kernel (N <= 64); None when the problem does not fit."""
         fn = getattr(lib(), "cubert_gemm_skinny_" + _suffix(C))
         rc = fn(self.handle, M, N, K, float(alpha), _ptr(A), lda, _ptr(B), ldb, _ptr(C), ldc, _ptr(bias), int(gelu))
         if rc == -2:
@@ -301,7 +301,8 @@ class Blas(object):
         return C
 
     def gemm_skinny_partials(self, M, N, K, A, lda, B, ldb, packed=False, partial_floats=1 << 20):
-        """A B left as K slices: (partials[slices, 32, pitch] fp32, slices, pitch); None when the problem does not fit."""
+        """A B left as K slices: (partials[slices, N rounded up to 32, pitch] fp32, slices, pitch); None when the
+        problem does not fit."""
         partials = torch.empty(partial_floats, dtype=torch.float32, device=B.device)
         slices, pitch = ctypes.c_int(0), ctypes.c_int(0)
         fn = getattr(lib(), "cubert_gemm_skinny_partials_" + _suffix(B))
@@ -310,7 +311,9 @@ class Blas(object):
         if rc == -2:
             return None
         _check(rc, fn.__name__)
-        return partials[:slices.value * 32 * pitch.value].view(slices.value, 32, pitch.value), slices.value, pitch.value
+        rows = (N + 31) // 32 * 32
+        return (partials[:slices.value * rows * pitch.value].view(slices.value, rows, pitch.value), slices.value,
+                pitch.value)
 
     def gemm_strided_batch(self, transA, transB, M, N, K, alpha, A, lda, sA, B, ldb, sB, beta, C, ldc, sC, batch):
         _call("cubert_gemm_strided_batch", C, self.handle, int(transA), int(transB), M, N, K, float(alpha), _ptr(A),

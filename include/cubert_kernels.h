@@ -70,16 +70,17 @@ int cubert_bias_res_ln_f16(cubert_half *inout, const cubert_half *residual, cons
                            const cubert_half *beta, const cubert_half *gamma, int rows, int hidden,
                            void *stream);
 
-/* cubert_bias_res_ln_* on a Dense output that cubert_gemm_skinny_partials_* left as K slices (at most 32 rows):
- *   a = storage type of (0.f + partials[(0 * 32 + r) * pitch + c] + partials[(1 * 32 + r) * pitch + c] + ...)
+/* cubert_bias_res_ln_* on a Dense output that cubert_gemm_skinny_partials_* left as K slices (at most 64 rows; R is
+ * `rows` rounded up to a multiple of 32, the token rows each slice holds):
+ *   a = storage type of (0.f + partials[(0 * R + r) * pitch + c] + partials[(1 * R + r) * pitch + c] + ...)
  *   x = a + bias + residual[r];  out[r] = beta + gamma * (x - mean) / sqrt(var + 1e-12)
  * i.e. cubert_gemm_skinny_* (alpha 1, no bias) followed by cubert_bias_res_ln_*, without the GEMM's hand-over between
- * workgroups.  Given the slices the result has the bits of cubert_bias_res_ln_* on their rounded sum, except for 768
- * halves, where cubert_bias_res_ln_f16 runs a kernel that adds a row's sums in another order (same inputs to the
- * LayerNorm, last-bit differences after it).  `out` is written only (it may be any buffer but `residual`).  Shapes the
+ * workgroups.  Given the slices, the fp32 result has the bits of cubert_bias_res_ln_f32 on their sum; in half
+ * precision the inputs to the LayerNorm are the same and a few results differ in the last bit (separately compiled
+ * kernels; at 768 halves cubert_bias_res_ln_f16 also adds a row's sums in another order).  `out` is written only (it may be any buffer but `residual`).  Shapes the
  * register-resident LayerNorm kernels do not take (hidden not 64 * {2,4,8} * {1..5}) return CUBERT_UNSUPPORTED
  * and launch nothing.
- * replaces: Dense + layer_norm_<T> of BertOutput / the attention output for a request of at most 32 tokens,
+ * replaces: Dense + layer_norm_<T> of BertOutput / the attention output for a request of at most 64 tokens,
  * reference src/cuBERT/op_att/Transformer.cpp:160-169 (op/Dense.cpp:47-57, op/LayerNorm.h:5-14). */
 int cubert_bias_res_ln_partials_f32(float *out, const float *partials, int slices, int pitch, const float *residual,
                                     const float *bias, const float *beta, const float *gamma, int rows, int hidden,
@@ -307,11 +308,13 @@ int cubert_bias_res_ln_split3_f32(float *inout, const float *residual, const flo
                                   const float *gamma, int rows, int hidden, float scale, cubert_half *split_out,
                                   int *overflow, void *stream);
 
-/* C = alpha * A * B + bias for N <= 32 columns (no transposes, beta = 0): the Dense layer of a request with at
- * most 32 tokens, where A is the [in, out] weight matrix (M = out, K = in) and each column of B one token.
- * One pass over the weights on the matrix cores with every load in flight at once; K is cut into slices that
- * are added in a fixed order, so results do not depend on scheduling.  cubert_gemm_* takes this path by
- * itself when the problem fits (CUBERT_GEMM=library in the environment turns that off).  Needs K a multiple
+/* C = alpha * A * B + bias for N <= 64 columns (no transposes, beta = 0): the Dense layer of a request with at
+ * most 64 tokens, where A is the [in, out] weight matrix (M = out, K = in) and each column of B one token.
+ * One pass over the weights on the matrix cores with every load in flight at once (from 33 tokens on a wavefront
+ * multiplies its weights with two blocks of 32 tokens); K is cut into slices that are added in a fixed order, so
+ * results do not depend on scheduling.  cubert_gemm_* takes this path by itself when the problem fits and
+ * N <= 32 (CUBERT_GEMM=library in the environment turns that off); beyond 32 tokens the library is the faster one
+ * for some shapes and the caller chooses (the host classes: see csrc/host/Transformer.cpp).  Needs K a multiple
  * of 16 and B 16-byte aligned with ldb a multiple of 16 bytes; anything else returns CUBERT_UNSUPPORTED and
  * launches nothing (also with CUBERT_GEMM=library or naive in the environment).  activation: 0 = none, 1 = the
  * erf-form GELU of cubert_bias_gelu applied to the result (Dense + bias + GELU of BertIntermediate in one
@@ -360,14 +363,15 @@ int cubert_gemm_skinny_packed_f16(void *handle, int M, int N, int K, float alpha
 /* The few-token product left as partial sums, for a consumer kernel that adds them while it loads its operand
  * (cubert_bias_res_ln_partials_*).  A few-token Dense kernel spends 2 of its 7-10 us
  * handing the K slices over to the workgroup that adds them; here every workgroup stores its slice and is done:
- *   partials[(slice * 32 + token) * pitch + feature] = sum over the slice's k of A[k, feature] * B[k, token]
- * for *slices slices, all 32 token rows (rows from N on are zero) and *pitch >= M features per row (fp32 whatever the
+ *   partials[(slice * R + token) * pitch + feature] = sum over the slice's k of A[k, feature] * B[k, token]
+ * for *slices slices, all R token rows (R = N rounded up to a multiple of 32; rows from N on are zero) and
+ * *pitch >= M features per row (fp32 whatever the
  * storage type; no alpha, bias or activation).  Adding the slices in slice order, starting from 0.f, and rounding
  * to the storage type is what a consumer does; the result is cubert_gemm_skinny_*'s for alpha = 1 and no bias up to
  * the order of the additions (the reduction may be cut into more slices here: nobody in this kernel has to add them,
  * and a weight matrix with few feature blocks streams faster when more workgroups pull on it).  packed != 0: A is the
  * output of cubert_gemm_skinny_pack_* (lda ignored).  partials must
- * hold partial_floats >= *slices * 32 * *pitch floats (1 << 20 is enough for every BERT-base/large Dense layer),
+ * hold partial_floats >= *slices * R * *pitch floats (1 << 20 is enough for every BERT-base/large Dense layer),
  * else CUBERT_UNSUPPORTED and nothing is launched; same conditions on K, B and ldb as cubert_gemm_skinny_*.
  * Asynchronous on the handle's stream.  No counterpart in the reference; same place as cubert_gemm_skinny_*
  * (src/cuBERT/op/Dense.cpp:47-57). */

@@ -870,9 +870,10 @@ def test_gemm_against_oracle_sgemm(K, name, ta, tb, M, N, K_):
 
 @pytest.mark.parametrize("name", ["f32", "f16"])
 @pytest.mark.parametrize("M,N,K_", [(768, 32, 768), (2304, 32, 768), (3072, 32, 768), (768, 32, 3072), (768, 1, 768),
-                                    (100, 7, 64), (33, 32, 16), (1024, 16, 4096), (2, 5, 768), (768, 32, 272)])
+                                    (100, 7, 64), (33, 32, 16), (1024, 16, 4096), (2, 5, 768), (768, 32, 272),
+                                    (768, 64, 768), (768, 33, 3072), (3072, 48, 768), (100, 50, 64), (1024, 64, 4096)])
 def test_gemm_skinny_against_oracle_sgemm(K, name, M, N, K_):
-    """Dense layer of a request with at most 32 tokens (column-major C[M,N] = A[M,K] B[K,N] + bias), K cut into
+    """Dense layer of a request with at most 64 tokens (column-major C[M,N] = A[M,K] B[K,N] + bias), K cut into
     1..16 slices; 30 launches in a row must give bit-identical results (slices are added in a fixed order and
     the arrival counters reset themselves)."""
     rng = np.random.default_rng(M + N + K_)
@@ -916,7 +917,7 @@ def test_gemm_skinny_against_oracle_sgemm(K, name, M, N, K_):
             assert torch.equal(C1, C2)
         else:
             assert_close(host(C2), host(C1), 2e-3, "packed vs plain weights, gelu=%s" % gelu)
-    # the general entry point takes the same path by itself
+    # the general entry point takes the same path by itself (up to 32 tokens; beyond, the library: same numbers)
     C = torch.zeros((N * M,), dtype=tdt(name), device="cuda")
     blas.gemm(0, 0, M, N, K_, 1.0, dA, M, dB, ldb, 0.0, C, M, bias=dbias)
     want = (oracle.sgemm(0, 0, M, N, K_, 1.0, A, M, B, ldb, 0.0, np.zeros(N * M, np.float32), M).reshape(N, M)
@@ -935,7 +936,8 @@ def _slices_added(partials, name):
 @pytest.mark.parametrize("name", ["f32", "f16"])
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("M,N,K_", [(768, 32, 768), (2304, 32, 768), (768, 32, 3072), (768, 1, 768), (100, 7, 64),
-                                    (1024, 16, 4096), (3072, 20, 1024), (33, 32, 16)])
+                                    (1024, 16, 4096), (3072, 20, 1024), (33, 32, 16), (768, 64, 768), (768, 40, 3072),
+                                    (1024, 64, 4096), (100, 33, 64)])
 def test_gemm_skinny_partials_add_up_to_the_gemm(K, name, packed, M, N, K_):
     """The few-token Dense product left as K slices: added in slice order and rounded they are what
     cubert_gemm_skinny_* stores (alpha 1, no bias) up to the order of the additions, rows from N on are zero, and a
@@ -952,7 +954,7 @@ def test_gemm_skinny_partials_add_up_to_the_gemm(K, name, packed, M, N, K_):
         got = blas.gemm_skinny_partials(M, N, K_, weights, M, dB, ldb, packed=packed)
         assert got is not None
         partials, slices, pitch = got
-        assert pitch >= M and pitch % 32 == 0 and slices >= 1
+        assert pitch >= M and pitch % 32 == 0 and slices >= 1 and partials.shape[1] == (N + 31) // 32 * 32
         C = torch.full((N * M,), 7.0, dtype=tdt(name), device="cuda")
         if packed:
             assert blas.gemm_skinny_packed(M, N, K_, 1.0, weights, dB, ldb, C, M) is not None
@@ -969,7 +971,7 @@ def test_gemm_skinny_partials_add_up_to_the_gemm(K, name, packed, M, N, K_):
 def test_gemm_skinny_partials_declines_what_it_cannot_do(K):
     blas = K.Blas()
     x = torch.zeros(64 * 1024, device="cuda")
-    assert blas.gemm_skinny_partials(64, 33, 64, x, 64, x, 64) is None             # more than 32 tokens
+    assert blas.gemm_skinny_partials(64, 65, 64, x, 64, x, 64) is None             # more than 64 tokens
     assert blas.gemm_skinny_partials(64, 8, 24, x, 64, x, 24) is None              # K not a multiple of 16
     assert blas.gemm_skinny_partials(64, 8, 32, x, 64, x[1:], 32) is None          # misaligned activations
     assert blas.gemm_skinny_partials(768, 8, 768, x, 768, x, 768, partial_floats=1000) is None  # buffer too small
@@ -979,7 +981,9 @@ def test_gemm_skinny_partials_declines_what_it_cannot_do(K):
 @pytest.mark.parametrize("name", ["f32", "f16"])
 @pytest.mark.parametrize("rows,hidden,in_features,with_bias", [(32, 768, 768, True), (32, 768, 3072, True),
                                                                (7, 768, 3072, False), (1, 1024, 4096, True),
-                                                               (20, 256, 1024, True), (32, 512, 64, False)])
+                                                               (20, 256, 1024, True), (32, 512, 64, False),
+                                                               (64, 768, 768, True), (33, 768, 3072, True),
+                                                               (50, 1024, 4096, False)])
 def test_bias_res_ln_from_partials_has_the_bits_of_layer_norm_of_the_added_slices(K, name, rows, hidden, in_features, with_bias):
     rng = np.random.default_rng(rows + hidden + in_features)
     blas = K.Blas()
@@ -995,11 +999,16 @@ def test_bias_res_ln_from_partials_has_the_bits_of_layer_norm_of_the_added_slice
     want = K.bias_res_ln_(C, residual, bias, beta, gamma)
     got = K.bias_res_ln_partials(partials, residual, bias, beta, gamma)
     assert got is not None
-    if name == "f32" or hidden != 768:
+    if name == "f32":
         assert torch.equal(got, want)
     else:
-        # 768 halves: bias_res_ln takes its two-rows-per-wavefront kernel there, whose row sums are added in another
-        # order; the values that go into the LayerNorm are the same
+        # half precision: the values that go into the LayerNorm are the same, but the two kernels are compiled
+        # separately (a multiply-add fused in one and not in the other moves a result across an fp16 rounding boundary
+        # now and then), and at 768 halves bias_res_ln takes its two-rows-per-wavefront kernel, whose row sums are
+        # added in another order: the last bit of a few elements
+        diff = (got.float() - want.float()).abs()
+        assert (diff <= want.float().abs() * 2.0 ** -9 + 1e-6).all()
+        assert (diff > 0).float().mean().item() < 0.01
         assert_close(host(got), host(want), 1e-3, "LayerNorm from partials against LayerNorm of the GEMM output")
     # and against the oracle's LayerNorm of the values the GEMM stored
     ref = oracle.layer_norm_(host(residual), dense_values + (host(bias) if with_bias else 0.0), host(beta), host(gamma))
@@ -1009,7 +1018,7 @@ def test_bias_res_ln_from_partials_has_the_bits_of_layer_norm_of_the_added_slice
 def test_bias_res_ln_from_partials_declines_what_it_cannot_do(K):
     partials = torch.zeros((3, 32, 768), device="cuda")
     v = torch.zeros(768, device="cuda")
-    assert K.bias_res_ln_partials(partials, torch.zeros((33, 768), device="cuda"), v, v, v) is None   # 33 rows
+    assert K.bias_res_ln_partials(partials, torch.zeros((65, 768), device="cuda"), v, v, v) is None   # 65 rows
     narrow = torch.zeros((3, 32, 128), device="cuda")
     assert K.bias_res_ln_partials(narrow, torch.zeros((4, 100), device="cuda"), v[:100], v[:100], v[:100]) is None  # hidden 100
     assert K.bias_res_ln_partials(narrow, torch.zeros((4, 768), device="cuda"), v, v, v) is None  # rows narrower than hidden
@@ -1018,7 +1027,7 @@ def test_bias_res_ln_from_partials_declines_what_it_cannot_do(K):
 def test_gemm_skinny_declines_what_it_cannot_do(K):
     blas = K.Blas()
     x = torch.zeros(64 * 1024, device="cuda")
-    assert blas.gemm_skinny(64, 33, 64, 1.0, x, 64, x, 64, x, 64) is None      # more than 32 tokens
+    assert blas.gemm_skinny(64, 65, 64, 1.0, x, 64, x, 64, x, 64) is None      # more than 64 tokens
     assert blas.gemm_skinny(64, 8, 24, 1.0, x, 64, x, 24, x, 64) is None       # K not a multiple of 16
     assert blas.gemm_skinny(64, 8, 32, 1.0, x, 64, x[1:], 32, x, 64) is None   # misaligned activations
     assert blas.gemm_skinny(64, 8, 32, 1.0, x, 64, x, 34, x, 64) is None       # row pitch not 16-byte aligned

@@ -140,6 +140,31 @@ def test_requests_of_at_most_32_tokens(cb, compute_type, seq_length):
         assert_close(full[k], want[k], tol, k)
 
 
+@pytest.mark.parametrize("compute_type", [0, 1])
+@pytest.mark.parametrize("seq_length,batches", [(32, (2,)), (64, (1,)), (16, (3, 4)), (8, (5, 8))])
+def test_requests_of_33_to_64_tokens(cb, compute_type, seq_length, batches):
+    """From 33 to 64 tokens the Dense layers in front of a LayerNorm (and, in half precision, the intermediate layer
+    with its GELU) still run on the few-token kernel, two blocks of 32 tokens per wavefront, the others on the
+    library: the request must match the oracle and itself as rows of a larger batch."""
+    from cubert_amd.testing import random_bert_weights, random_inputs
+    w = random_bert_weights(seed=21, labels=2, pooler=True, classifier=True, ln_random=True, **SMALL)
+    total = 160 // seq_length
+    ids, mask, seg = random_inputs(seed=22, batch=total, seq_length=seq_length, vocab=SMALL["vocab"], min_valid=3,
+                                   segment_split=5)
+    tol = FP16_TOL if compute_type else FP32_TOL
+    wo = {k: oracle.round_to_half(v) for k, v in w.items()} if compute_type else w
+    want = oracle.bert_forward(wo, ids, mask, seg, 3, 4)
+    bert = cb.Bert(w, total, seq_length, 3, 4, compute_type)
+    full = bert.forward(ids, mask, seg)
+    for n in batches:
+        assert 32 < n * seq_length <= 64
+        few = bert.forward(ids[:n], mask[:n], seg[:n])
+        for k in ("sequence_output", "pooled_output", "logits", "probs"):
+            assert_close(few[k], want[k][:n], tol, "%s, %d request(s) of %d tokens" % (k, n, seq_length))
+            assert_close(few[k], full[k][:n], tol, "%s vs the same rows of a batch of %d" % (k, total))
+    bert.close()
+
+
 def test_repeated_calls_and_smaller_batches_reuse_buffers(cb):
     """The reference's BertMTest calls one model four times; results must not depend on what ran before."""
     from cubert_amd.testing import random_bert_weights, random_inputs

@@ -94,6 +94,7 @@ def test_two_calls_in_a_row_the_second_smaller(L, context):
     # BERT-base feed-forward shapes at 32 tokens (K cut into slices: partial tiles and counters in use), then a
     # smaller problem that reuses the front of the same scratch
     run_pair(L, handle, stream, 3072, 32, 768, 1, seed=1)
+    run_pair(L, handle, stream, 768, 64, 3072, 0, seed=6)      # two blocks of 32 tokens per wavefront
     run_pair(L, handle, stream, 768, 32, 3072, 0, seed=2)
     run_pair(L, handle, stream, 96, 5, 256, 0, seed=3)
     run_pair(L, handle, stream, 768, 32, 768, 0, seed=4, with_bias=False)
@@ -123,13 +124,13 @@ def test_calls_leave_free_device_memory_unchanged(L, context):
     # first launch is the runtime's business, not this entry point's
     assert call(M, N, K) == 0
     assert call(96, 5, 256) == 0
-    assert call(32, 33, 16) == UNSUPPORTED
+    assert call(32, 65, 16) == UNSUPPORTED
     assert L.cubert_stream_synchronize(stream) == 0
     before = free_device_bytes(L)
     for _ in range(20):
         assert call(M, N, K) == 0
         assert call(96, 5, 256) == 0
-        assert call(32, 33, 16) == UNSUPPORTED
+        assert call(32, 65, 16) == UNSUPPORTED
     assert call(NOALLOC_MAX_M + 1, 1, 16) == TOO_LARGE
     assert L.cubert_stream_synchronize(stream) == 0
     assert free_device_bytes(L) == before
@@ -169,7 +170,7 @@ def test_sizes_beyond_the_fixed_scratch_are_refused(L, context, capfd):
     assert L.cubert_gemm_skinny_noalloc_f32(stream, 32, 1, NOALLOC_MAX_K + 16, 1.0, p, 32, p, NOALLOC_MAX_K + 16, p, 32,
                                             None, 0) == TOO_LARGE
     assert L.cubert_gemm_skinny_noalloc_f32(stream, 32, 1, 16, 1.0, None, 32, p, 16, p, 32, None, 0) == BAD_ARGUMENT
-    assert L.cubert_gemm_skinny_noalloc_f32(stream, 32, 33, 16, 1.0, p, 32, p, 16, p, 32, None, 0) == UNSUPPORTED
+    assert L.cubert_gemm_skinny_noalloc_f32(stream, 32, 65, 16, 1.0, p, 32, p, 16, p, 32, None, 0) == UNSUPPORTED
     assert L.cubert_gemm_skinny_noalloc_f32(stream, 32, 1, 24, 1.0, p, 32, p, 24, p, 32, None, 0) == UNSUPPORTED
     assert L.cubert_stream_synchronize(stream) == 0
     d.free()
