@@ -183,6 +183,12 @@ int build_plan(BlasContext *ctx, const GemmKey &k, GemmPlan *plan) {
 // decision as its GEMM_ALGO_* environment variables, src/cuBERT/common.cpp:106-160.)
 
 constexpr double kTuneMinFlops = 1e9;
+// fp32 operands are timed from much smaller shapes on (forward pass of BERT-base fp32 at seq 32 with against without,
+// two alternating runs on one box: batch 4 0.740 / 0.757 ms, batch 6 0.791 / 0.898, batch 8 0.887 / 0.943, batch 16
+// 1.110 / 1.184, batch 32 1.71-1.75 / 1.829; batch 3 equal).  The same for fp16 operands loses more often than it
+// wins (batch 4 0.565 / 0.546 ms, batch 6 0.56-0.59 / 0.54-0.56, batch 8 0.56-0.58 / 0.55), so they keep the limits.
+constexpr double kTuneMinFlopsF32 = 5e7;
+constexpr float kTuneMinCallMsF32 = 0.004f;
 constexpr int kTuneRuns = 8;
 constexpr int kTunePasses = 2;
 constexpr float kTuneMinGain = 0.99f;  // leave the heuristic's first choice unless another is at least 1 % faster
@@ -213,7 +219,10 @@ std::map<GemmKey, int> &tuned_ranks() {
 void tune_plan(BlasContext *ctx, const GemmKey &k, GemmPlan &p, float alpha, const void *A, const void *B, void *C) {
     p.tuned = true;
     const double flops = 2.0 * k.M * k.N * k.K * k.batch;
-    if (!tuning_enabled() || !k.beta_zero || p.candidates.size() < 2 || flops < kTuneMinFlops) return;
+    const bool f32 = k.type == 0;
+    if (!tuning_enabled() || !k.beta_zero || p.candidates.size() < 2 || flops < (f32 ? kTuneMinFlopsF32 : kTuneMinFlops)) {
+        return;
+    }
     {
         std::lock_guard<std::mutex> lock(tuned_mutex());
         auto it = tuned_ranks().find(k);
@@ -262,7 +271,7 @@ void tune_plan(BlasContext *ctx, const GemmKey &k, GemmPlan &p, float alpha, con
                 continue;
             }
             if (fastest[i] == 0.f || ms < fastest[i]) fastest[i] = ms;
-            if (pass == 0 && i == 0 && ms < kTuneMinCallMs * kTuneRuns) {
+            if (pass == 0 && i == 0 && ms < (f32 ? kTuneMinCallMsF32 : kTuneMinCallMs) * kTuneRuns) {
                 std::lock_guard<std::mutex> lock(tuned_mutex());
                 tuned_ranks()[k] = 0;
                 return;
